@@ -1,0 +1,241 @@
+// C ABI of libesmoe.so: argument checks, schedule policy, kernel launches.
+// Declarations and the reference entry points they replace: include/esmoe.h.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "esmoe.h"
+#include "gemm_args.h"
+#include "schedule.h"
+
+extern "C" int esmoe_launch_grouped_gemm(const esmoe::GemmArgs* args, int mx, int grid, hipStream_t stream);
+extern "C" int esmoe_launch_mxfp8_quant(const void* in, int in_dtype, const int* problem_sizes,
+                                        const int* expert_offsets, const int* blockscale_offsets, void* q, uint8_t* sf,
+                                        int num_experts, int sf_rows, int k, hipStream_t stream);
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+struct DeviceInfo {
+  int valid = 0;
+  int cus = 0;
+  int is_gfx950 = 0;
+};
+DeviceInfo g_dev[64];
+std::mutex g_dev_mu;
+
+// Properties of the current device, queried once per device.
+int current_device_info(DeviceInfo* out) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail((int)err, "hipGetDevice failed: %s", hipGetErrorString(err));
+  if (dev < 0 || dev >= 64) return fail(ESMOE_ERR_UNSUPPORTED_DEVICE, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_dev_mu);
+  if (!g_dev[dev].valid) {
+    hipDeviceProp_t prop;
+    err = hipGetDeviceProperties(&prop, dev);
+    if (err != hipSuccess) return fail((int)err, "hipGetDeviceProperties failed: %s", hipGetErrorString(err));
+    g_dev[dev].cus = prop.multiProcessorCount;
+    g_dev[dev].is_gfx950 = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    g_dev[dev].valid = 1;
+  }
+  *out = g_dev[dev];
+  if (!out->is_gfx950) return fail(ESMOE_ERR_UNSUPPORTED_DEVICE, "libesmoe kernels are built for gfx950 only");
+  return 0;
+}
+
+int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v && *v ? atoi(v) : dflt;
+}
+
+// Default schedule policy; ESMOE_* environment variables override single fields (tuning aid).
+esmoe::SchedPolicy make_policy(int force_bm) {
+  esmoe::SchedPolicy p;
+  p.force_mt = force_bm / 16;
+  p.big_mt = env_int("ESMOE_BIG_MT", 8);
+  p.nt_light = env_int("ESMOE_NT_LIGHT", 4);
+  p.nt_heavy = env_int("ESMOE_NT_HEAVY", 4);
+  p.light_max_mt = env_int("ESMOE_LIGHT_MAX_MT", 4);
+  p.order = env_int("ESMOE_ORDER", 0);
+  if (p.force_mt == 16 || p.big_mt == 16) p.nt_heavy = 2;  // the 256-row tile exists 128 columns wide only
+  if (p.force_mt && p.force_mt > p.light_max_mt && p.force_mt < 16 && p.nt_heavy == 1) p.nt_heavy = 2;
+  return p;
+}
+
+int check_common(const void* out, const void* a, const void* b, const int32_t* ps, const int32_t* eo, int num_experts,
+                 int total_rows, int n, int k, int force_bm, void* workspace, size_t workspace_bytes, int out_dtype) {
+  if (!out || !a || !b || !ps || !eo) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if (num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "num_experts must be in [1, %d], got %d", ESMOE_MAX_EXPERTS, num_experts);
+  if (n <= 0 || n % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "n must be a positive multiple of 128, got %d", n);
+  if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must be a positive multiple of 128, got %d", k);
+  if (total_rows < 0) return fail(ESMOE_ERR_INVALID_ARGUMENT, "total_rows must be >= 0");
+  if (out_dtype != ESMOE_OUT_BF16 && out_dtype != ESMOE_OUT_FP16)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "out_dtype must be ESMOE_OUT_BF16 or ESMOE_OUT_FP16");
+  if (force_bm != 0 && force_bm != 16 && force_bm != 32 && force_bm != 64 && force_bm != 128 && force_bm != 256)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "force_bm must be 0, 16, 32, 64, 128 or 256, got %d", force_bm);
+  if (!workspace || workspace_bytes < esmoe_gemm_workspace_bytes(num_experts))
+    return fail(ESMOE_ERR_WORKSPACE_TOO_SMALL, "workspace of %zu bytes is smaller than the %zu required",
+                workspace_bytes, esmoe_gemm_workspace_bytes(num_experts));
+  if ((uintptr_t)workspace % 4) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace must be 4-byte aligned");
+  if ((uintptr_t)a % 16 || (uintptr_t)b % 16 || (uintptr_t)out % 8)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "a and b must be 16-byte aligned, out 8-byte aligned");
+  return 0;
+}
+
+int launch_gemm(esmoe::GemmArgs& g, int mx, int force_bm, void* stream) {
+  if (g.total_rows == 0) return 0;
+  DeviceInfo info;
+  int rc = current_device_info(&info);
+  if (rc) return rc;
+  g.policy = make_policy(force_bm);
+  int grid = info.cus * env_int("ESMOE_WGS_PER_CU", 1);
+  rc = esmoe_launch_grouped_gemm(&g, mx, grid, (hipStream_t)stream);
+  if (rc) return fail(rc, "grouped GEMM launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t esmoe_gemm_workspace_bytes(int num_experts) {
+  if (num_experts < 0) num_experts = 0;
+  size_t bytes = (size_t)esmoe::ws_words(num_experts) * 4;
+  return (bytes + 255) & ~(size_t)255;
+}
+
+int esmoe_fp8_blockwise_grouped_mm(void* out, int out_dtype, const void* a, const void* b, const float* sa,
+                                   const float* sb, const int32_t* problem_sizes, const int32_t* expert_offsets,
+                                   int num_experts, int total_rows, int n, int k, int force_bm, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int rc = check_common(out, a, b, problem_sizes, expert_offsets, num_experts, total_rows, n, k, force_bm, workspace,
+                        workspace_bytes, out_dtype);
+  if (rc) return rc;
+  if (!sa || !sb) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null scale pointer");
+  esmoe::GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.b = b; g.sa = sa; g.sb = sb; g.out = out;
+  g.problem_sizes = problem_sizes; g.expert_offsets = expert_offsets;
+  g.ws = (int32_t*)workspace;
+  g.num_experts = num_experts; g.total_rows = total_rows; g.n = n; g.k = k; g.out_dtype = out_dtype;
+  return launch_gemm(g, 0, force_bm, stream);
+}
+
+int esmoe_mxfp8_grouped_mm(void* d, int out_dtype, const void* a, const void* b, const uint8_t* sfa,
+                           const uint8_t* sfb, const int32_t* problem_sizes, const int32_t* expert_offsets,
+                           const int32_t* blockscale_offsets, int num_experts, int total_rows, int n, int k,
+                           int force_bm, void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int rc = check_common(d, a, b, problem_sizes, expert_offsets, num_experts, total_rows, n, k, force_bm, workspace,
+                        workspace_bytes, out_dtype);
+  if (rc) return rc;
+  if (!sfa || !sfb || !blockscale_offsets) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null scale pointer");
+  if ((uintptr_t)sfa % 4 || (uintptr_t)sfb % 4)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "sfa and sfb must be 4-byte aligned");
+  esmoe::GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.b = b; g.sfa = sfa; g.sfb = sfb; g.out = d;
+  g.problem_sizes = problem_sizes; g.expert_offsets = expert_offsets; g.blockscale_offsets = blockscale_offsets;
+  g.ws = (int32_t*)workspace;
+  g.num_experts = num_experts; g.total_rows = total_rows; g.n = n; g.k = k; g.out_dtype = out_dtype;
+  return launch_gemm(g, 1, force_bm, stream);
+}
+
+int esmoe_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* problem_sizes,
+                              const int32_t* expert_offsets, const int32_t* blockscale_offsets, void* q,
+                              uint8_t* sf, int num_experts, int total_rows, int sf_rows, int k, void* stream) {
+  g_err[0] = 0;
+  if (!in || !problem_sizes || !expert_offsets || !blockscale_offsets || !q || !sf)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if (num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "num_experts must be in [1, %d], got %d", ESMOE_MAX_EXPERTS, num_experts);
+  if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must align to 128, got %d", k);
+  if (in_dtype != ESMOE_IN_BF16 && in_dtype != ESMOE_IN_FP16)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in_dtype must be ESMOE_IN_BF16 or ESMOE_IN_FP16");
+  if (total_rows < 0 || sf_rows < 0 || sf_rows % 128)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "sf_rows must be a non-negative multiple of 128, got %d", sf_rows);
+  if ((uintptr_t)in % 16 || (uintptr_t)q % 8 || (uintptr_t)sf % 16)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in and sf must be 16-byte aligned, q 8-byte aligned");
+  if (total_rows == 0 || sf_rows == 0) return 0;
+  DeviceInfo info;
+  int rc = current_device_info(&info);
+  if (rc) return rc;
+  rc = esmoe_launch_mxfp8_quant(in, in_dtype, problem_sizes, expert_offsets, blockscale_offsets, q, sf, num_experts,
+                                sf_rows, k, (hipStream_t)stream);
+  if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return 0;
+}
+
+int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int32_t* ws_host) {
+  g_err[0] = 0;
+  if (!problem_sizes_host || !ws_host || num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS || n <= 0 || n % 128)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_schedule");
+  const esmoe::SchedPolicy p = make_policy(force_bm);
+  int32_t* item_start = ws_host + esmoe::ws_item_start(num_experts);
+  int32_t* order = ws_host + esmoe::ws_order(num_experts);
+  // same ranking as the device schedule kernel: most rows first, ties by expert index
+  for (int e = 0; e < num_experts; e++) {
+    int m = problem_sizes_host[e * 3] < 0 ? 0 : problem_sizes_host[e * 3];
+    int pos = e;
+    if (p.order == 0) {
+      pos = 0;
+      for (int j = 0; j < num_experts; j++) {
+        int mj = problem_sizes_host[j * 3] < 0 ? 0 : problem_sizes_host[j * 3];
+        pos += (mj > m) || (mj == m && j < e);
+      }
+    }
+    order[pos] = e;
+  }
+  int run = 0;
+  for (int pos = 0; pos < num_experts; pos++) {
+    int m = problem_sizes_host[order[pos] * 3];
+    item_start[pos] = run;
+    run += esmoe::sched_items(m, n, p);
+  }
+  item_start[num_experts] = run;
+  ws_host[esmoe::kWsTotal] = run;
+  ws_host[esmoe::kWsCounter] = 0;
+  return 0;
+}
+
+int esmoe_host_decode_item(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
+                           int force_bm, int item, int32_t* out5) {
+  g_err[0] = 0;
+  if (!problem_sizes_host || !ws_host || !out5) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null pointer");
+  const esmoe::SchedPolicy p = make_policy(force_bm);
+  const int32_t* item_start = ws_host + esmoe::ws_item_start(num_experts);
+  const int32_t* order = ws_host + esmoe::ws_order(num_experts);
+  if (item < 0 || item >= ws_host[esmoe::kWsTotal]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "item out of range");
+  int lo = 0, hi = num_experts;
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (item_start[mid] <= item) lo = mid; else hi = mid;
+  }
+  const int e = order[lo];
+  const esmoe::TileCoord t = esmoe::sched_decode(item - item_start[lo], problem_sizes_host[e * 3], n, p);
+  out5[0] = e; out5[1] = t.mt * 16; out5[2] = t.nt * 64; out5[3] = t.m0; out5[4] = t.n0;
+  return 0;
+}
+
+const char* esmoe_last_error(void) { return g_err; }
+
+const char* esmoe_version(void) { return "esmoe 0.1 (gfx950)"; }
+
+}  // extern "C"

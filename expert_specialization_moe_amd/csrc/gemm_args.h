@@ -1,0 +1,29 @@
+// Kernel argument block shared by the host launcher and the grouped GEMM kernels.
+#pragma once
+#include <stdint.h>
+
+#include "schedule.h"
+
+namespace esmoe {
+
+struct GemmArgs {
+  const void* a;        // [total_rows, K] e4m3
+  const void* b;        // [E, N, K] e4m3
+  const float* sa;      // fp8-blockwise: [total_rows, K/128]
+  const float* sb;      // fp8-blockwise: [E, N/128, K/128]
+  const uint8_t* sfa;   // mxfp8: swizzled E8M0, expert base blockscale_offsets[e] * K/32
+  const uint8_t* sfb;   // mxfp8: swizzled E8M0, expert base e * N * K/32
+  void* out;            // [total_rows, N]
+  const int32_t* problem_sizes;
+  const int32_t* expert_offsets;
+  const int32_t* blockscale_offsets;
+  int32_t* ws;          // schedule workspace, ws_words(num_experts) int32
+  int num_experts;
+  int total_rows;
+  int n;
+  int k;
+  int out_dtype;        // 0 bf16, 1 fp16
+  SchedPolicy policy;
+};
+
+}  // namespace esmoe

@@ -1,0 +1,130 @@
+// MXFP8 grouped quantisation for gfx950: bf16/fp16 rows -> e4m3 bytes + swizzled E8M0 scales.
+//
+// Arithmetic follows cvt_warp_fp16_to_mxfp8
+// (expert_specialization/csrc/cuda/es_sm100_mxfp8_blockscaled_group_quant.cuh:36-134):
+// per 1x32 block  amax = max|x|,  scale = smallest power of two >= amax/448,
+// q = e4m3_rne(x / scale).  The scale exponent is taken from the bit pattern of
+// amax (448 = 1.75 * 2^8  =>  E = exponent(amax) - 8 + (mantissa > .75)), which equals
+// the reference's float route with a correctly rounded 1/448.
+//
+// Work decomposition: one workgroup per 128-row x 128-column tile of the *scale*
+// row space (blockscale_offsets are multiples of 128, so a tile belongs to one
+// expert).  16 lanes read one row of the tile (16 bytes each, a 256-byte coalesced
+// segment), 4 lanes share one 32-wide block and reduce amax with two lane swaps.
+// The 512-byte scale tile (128 rows x 4 scale columns, layout ((32,4),4):((16,4),1),
+// group_quant.cuh:25) is assembled in LDS and written with 16-byte stores.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace esmoe {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+constexpr int kQuantThreads = 256;
+
+template <bool FP16>
+__device__ __forceinline__ void unpack8(v4i raw, float* x) {
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    uint32_t w = (uint32_t)raw[i];
+    if constexpr (FP16) {
+      x[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+      x[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+    } else {
+      x[2 * i] = __builtin_bit_cast(float, w << 16);
+      x[2 * i + 1] = __builtin_bit_cast(float, w & 0xffff0000u);
+    }
+  }
+}
+
+// E8M0 code of the smallest power of two >= amax / 448 (amax >= 0, finite).
+__device__ __forceinline__ int mx_scale_code(float amax) {
+  uint32_t bits = __builtin_bit_cast(uint32_t, amax);
+  int code = (int)((bits >> 23) & 0xff) - 8 + ((bits & 0x7fffffu) > 0x600000u ? 1 : 0);
+  code = code < 0 ? 0 : (code > 254 ? 254 : code);
+  return amax == 0.f ? 0 : code;
+}
+
+template <bool FP16>
+__global__ void __launch_bounds__(kQuantThreads) mxfp8_quant_kernel(const uint16_t* __restrict__ in,
+                                                                    const int* __restrict__ problem_sizes,
+                                                                    const int* __restrict__ expert_offsets,
+                                                                    const int* __restrict__ blockscale_offsets,
+                                                                    uint8_t* __restrict__ q, uint8_t* __restrict__ sf,
+                                                                    int num_experts, int k) {
+  __shared__ __attribute__((aligned(16))) uint8_t s_sf[512];
+  const int kt = blockIdx.x;               // 128-column tile
+  const int sf_row0 = blockIdx.y * 128;    // first row of this tile in scale-row space
+  const int tid = threadIdx.x;
+
+  // expert owning scale row sf_row0: last e with blockscale_offsets[e] <= sf_row0
+  int lo = 0, hi = num_experts;
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (blockscale_offsets[mid] <= sf_row0) lo = mid; else hi = mid;
+  }
+  const int e = lo;
+  const int m_e = problem_sizes[e * 3];
+  const int r0 = sf_row0 - blockscale_offsets[e];  // first row of the tile inside the expert
+  if (r0 < 0 || r0 >= m_e) return;                 // tile past the expert's rows: nothing defined there
+  const long row_base = expert_offsets[e];
+  const int kcols = k >> 5;
+
+  const int sub = tid & 15;        // 16-byte column of the row: elements [8*sub, 8*sub + 8)
+  const int rrow = tid >> 4;       // row within a 16-row pass
+  v4i raw[8];
+#pragma unroll
+  for (int p = 0; p < 8; p++) {
+    int r = r0 + p * 16 + rrow;
+    raw[p] = v4i{0, 0, 0, 0};
+    if (r < m_e) raw[p] = __builtin_nontemporal_load((const v4i*)(in + (row_base + r) * k + kt * 128 + sub * 8));
+  }
+#pragma unroll
+  for (int p = 0; p < 8; p++) {
+    const int rt = p * 16 + rrow;  // row within the tile
+    const int r = r0 + rt;
+    float x[8];
+    unpack8<FP16>(raw[p], x);
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) amax = __builtin_fmaxf(amax, __builtin_fabsf(x[i]));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 1));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 2));
+    const int code = mx_scale_code(amax);
+    const float inv = amax == 0.f ? 0.f : __builtin_bit_cast(float, (uint32_t)(254 - code) << 23);
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) y[i] = __builtin_amdgcn_fmed3f(x[i] * inv, -448.f, 448.f);
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], 0, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+    if (r < m_e) {
+      __builtin_nontemporal_store(v2i{w0, w1}, (v2i*)(q + (row_base + r) * k + kt * 128 + sub * 8));
+    }
+    if ((sub & 3) == 0) s_sf[(rt & 31) * 16 + (rt >> 5) * 4 + (sub >> 2)] = (uint8_t)(r < m_e ? code : 0);
+  }
+  __syncthreads();
+  if (tid < 32) {
+    uint8_t* dst = sf + (long)blockscale_offsets[e] * kcols + ((long)(r0 >> 7) * (k >> 7) + kt) * 512;
+    *(v4i*)(dst + tid * 16) = *(const v4i*)(s_sf + tid * 16);
+  }
+}
+
+}  // namespace esmoe
+
+extern "C" int esmoe_launch_mxfp8_quant(const void* in, int in_dtype, const int* problem_sizes,
+                                        const int* expert_offsets, const int* blockscale_offsets, void* q, uint8_t* sf,
+                                        int num_experts, int sf_rows, int k, hipStream_t stream) {
+  using namespace esmoe;
+  dim3 grid(k / 128, sf_rows / 128);
+  if (grid.x == 0 || grid.y == 0) return 0;
+  if (in_dtype == 1)
+    hipLaunchKernelGGL(mxfp8_quant_kernel<true>, grid, dim3(kQuantThreads), 0, stream, (const uint16_t*)in,
+                       problem_sizes, expert_offsets, blockscale_offsets, (uint8_t*)q, sf, num_experts, k);
+  else
+    hipLaunchKernelGGL(mxfp8_quant_kernel<false>, grid, dim3(kQuantThreads), 0, stream, (const uint16_t*)in,
+                       problem_sizes, expert_offsets, blockscale_offsets, (uint8_t*)q, sf, num_experts, k);
+  return (int)hipGetLastError();
+}

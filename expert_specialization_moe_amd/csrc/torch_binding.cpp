@@ -1,0 +1,240 @@
+// PyTorch-ROCm operator registration for the three expert_specialization ops.
+//
+// Same library name, schemas and dispatch key as the reference
+// (expert_specialization/csrc/expert_specialization.cpp:56-73); the argument
+// checks mirror its TORCH_CHECKs (es_fp8_blockwise.cu:47-56,
+// es_sm100_mxfp8_blockscaled.cu:15-25, es_sm100_mxfp8_blockscaled_group_quant.cu:13-24,
+// es_fp8_blockwise_launcher.cuh:53).  Everything below the checks is the C ABI of
+// libesmoe.so (include/esmoe.h): this file only unwraps tensors.
+//
+// Validation is also registered for CPU tensors so that it can be exercised on a
+// machine without a GPU; after the checks pass a CPU call fails loudly, there is
+// no CPU implementation of the ops.
+#include <Python.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/all.h>
+
+#include "esmoe.h"
+
+extern "C" {
+// Empty module so that `import ..._C` loads this library and runs the static
+// registrations below (same device as the reference, expert_specialization.cpp:4-21).
+PyObject* PyInit__C(void) {
+  static struct PyModuleDef module_def = {PyModuleDef_HEAD_INIT, "_C", NULL, -1, NULL};
+  return PyModule_Create(&module_def);
+}
+}
+
+namespace {
+
+void* current_stream(const torch::Tensor& t) {
+  return (void*)c10::hip::getCurrentHIPStream(t.device().index()).stream();
+}
+
+void require_device(const torch::Tensor& t, const char* op) {
+  TORCH_CHECK(t.is_cuda(), op, ": tensors must live on a HIP device (MI355X); there is no CPU implementation");
+}
+
+void check_rc(int rc, const char* op) { TORCH_CHECK(rc == 0, op, " failed (", rc, "): ", esmoe_last_error()); }
+
+int out_dtype_of(const torch::Tensor& t) { return t.scalar_type() == torch::kBFloat16 ? ESMOE_OUT_BF16 : ESMOE_OUT_FP16; }
+
+// Scratch for the device-built schedule: the caller's workspace when it is big
+// enough and aligned, otherwise a small tensor from the caching allocator.
+torch::Tensor schedule_scratch(const torch::Tensor* workspace, int64_t num_experts, const torch::Tensor& like) {
+  const int64_t need = (int64_t)esmoe_gemm_workspace_bytes((int)num_experts);
+  if (workspace && workspace->defined() && workspace->is_cuda() && workspace->is_contiguous() &&
+      workspace->nbytes() >= (size_t)need && (reinterpret_cast<uintptr_t>(workspace->data_ptr()) % 16) == 0) {
+    return *workspace;
+  }
+  return torch::empty({need}, torch::TensorOptions().dtype(torch::kUInt8).device(like.device()));
+}
+
+}  // namespace
+
+void es_fp8_blockwise_scaled_grouped_mm(torch::Tensor& output, const torch::Tensor& a, const torch::Tensor& b,
+                                        const torch::Tensor& scales_a, const torch::Tensor& scales_b,
+                                        const torch::Tensor& stride_a, const torch::Tensor& stride_b,
+                                        const torch::Tensor& stride_d, const torch::Tensor& problem_sizes,
+                                        const torch::Tensor& expert_offsets, const torch::Tensor& workspace) {
+  TORCH_CHECK(problem_sizes.dim() == 2, "problem_sizes must be 2D tensor");
+  TORCH_CHECK(problem_sizes.size(1) == 3, "problem_sizes must have shape (num_experts, 3)");
+  TORCH_CHECK(problem_sizes.size(0) == expert_offsets.size(0),
+              "Number of experts in problem_sizes must match expert_offsets");
+  TORCH_CHECK(problem_sizes.dtype() == torch::kInt32, "problem_sizes must be int32");
+  TORCH_CHECK(expert_offsets.dtype() == torch::kInt32, "expert_offsets must be int32");
+  TORCH_CHECK(a.scalar_type() == torch::kFloat8_e4m3fn, "a must be kFloat8_e4m3fn");
+  TORCH_CHECK(b.scalar_type() == torch::kFloat8_e4m3fn, "b must be kFloat8_e4m3fn");
+  TORCH_CHECK(output.scalar_type() == torch::kBFloat16 || output.scalar_type() == torch::kHalf,
+              "output must be bfloat16 or half");
+  const int64_t num_experts = problem_sizes.size(0);
+  TORCH_CHECK(num_experts >= 1 && num_experts <= ESMOE_MAX_EXPERTS, "Number of experts cannot exceed 1024");
+  // Layout contract (the reference only ever dereferences data_ptr(), so the views below are the
+  // ones its callers build: test/test_es_grouped_gemm.py:145-170).
+  TORCH_CHECK(a.dim() == 2 && a.stride(1) == 1 && a.stride(0) == a.size(1), "a must be a packed row-major (rows, k) tensor");
+  TORCH_CHECK(b.dim() == 3 && b.size(0) == num_experts, "b must be a (num_experts, k, n) tensor");
+  TORCH_CHECK(b.stride(1) == 1 && b.stride(2) == b.size(1) && b.stride(0) == b.size(1) * b.size(2),
+              "b must be the column-major (num_experts, k, n) view of a packed (num_experts, n, k) tensor");
+  const int64_t total_rows = a.size(0), k = a.size(1), n = b.size(2);
+  TORCH_CHECK(b.size(1) == k, "a and b disagree on k");
+  TORCH_CHECK(k % 128 == 0 && n % 128 == 0, "n and k must be multiples of 128");
+  TORCH_CHECK(output.dim() == 2 && output.size(0) == total_rows && output.size(1) == n && output.is_contiguous(),
+              "output must be a contiguous (rows, n) tensor");
+  TORCH_CHECK(scales_a.scalar_type() == torch::kFloat32 && scales_b.scalar_type() == torch::kFloat32,
+              "scales must be float32");
+  TORCH_CHECK(scales_a.dim() == 2 && scales_a.size(0) == total_rows && scales_a.size(1) == k / 128 &&
+                  scales_a.is_contiguous(),
+              "scales_a must be a contiguous (rows, k/128) tensor");
+  TORCH_CHECK(scales_b.dim() == 3 && scales_b.size(0) == num_experts && scales_b.size(1) == k / 128 &&
+                  scales_b.size(2) == n / 128 && scales_b.stride(1) == 1 &&
+                  (scales_b.size(2) == 1 || scales_b.stride(2) == k / 128),
+              "scales_b must be the (num_experts, k/128, n/128) view of a packed (num_experts, n/128, k/128) tensor");
+  for (const torch::Tensor* s : {&stride_a, &stride_b, &stride_d}) {
+    TORCH_CHECK(s->dim() == 1 && s->size(0) == num_experts, "stride tensors must have one entry per expert");
+  }
+  TORCH_CHECK(total_rows < (int64_t(1) << 31) && n < (int64_t(1) << 31) && k < (int64_t(1) << 31), "tensor too large");
+
+  require_device(a, "es_fp8_blockwise_scaled_grouped_mm");
+  for (const torch::Tensor* t :
+       {(const torch::Tensor*)&output, &b, &scales_a, &scales_b, &problem_sizes, &expert_offsets}) {
+    TORCH_CHECK(t->device() == a.device(), "all tensors must be on the same device");
+  }
+  TORCH_CHECK(problem_sizes.is_contiguous() && expert_offsets.is_contiguous(), "metadata tensors must be contiguous");
+  if (total_rows == 0) return;
+  c10::DeviceGuard guard(a.device());
+  torch::Tensor ws = schedule_scratch(&workspace, num_experts, a);
+  int rc = esmoe_fp8_blockwise_grouped_mm(
+      output.data_ptr(), out_dtype_of(output), a.data_ptr(), b.data_ptr(), scales_a.data_ptr<float>(),
+      scales_b.data_ptr<float>(), problem_sizes.data_ptr<int32_t>(), expert_offsets.data_ptr<int32_t>(),
+      (int)num_experts, (int)total_rows, (int)n, (int)k, /*force_bm=*/0, ws.data_ptr(), ws.nbytes(), current_stream(a));
+  check_rc(rc, "es_fp8_blockwise_scaled_grouped_mm");
+}
+
+void es_sm100_mxfp8_blockscaled_grouped_mm(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& sfa,
+                                           const torch::Tensor& sfb, torch::Tensor& d,
+                                           const torch::Tensor& problem_sizes, const torch::Tensor& expert_offsets,
+                                           const torch::Tensor& blockscale_offsets) {
+  TORCH_CHECK(problem_sizes.dim() == 2, "problem_sizes must be 2D tensor");
+  TORCH_CHECK(problem_sizes.size(1) == 3, "problem_sizes must have shape (num_experts, 3)");
+  TORCH_CHECK(problem_sizes.size(0) == expert_offsets.size(0),
+              "Number of experts in problem_sizes must match expert_offsets");
+  TORCH_CHECK(problem_sizes.dtype() == torch::kInt32, "problem_sizes must be int32");
+  TORCH_CHECK(a.dim() == 2, "a must be a 2D tensor of shape (num_tokens, k)");
+  TORCH_CHECK(b.dim() == 3, "b must be a 3D tensor of shape (num_experts, k, n)");
+  TORCH_CHECK(a.size(1) == b.size(1) && a.size(1) % 128 == 0, "k should align 128");
+  TORCH_CHECK(b.size(2) % 128 == 0, "n should align 128");
+  TORCH_CHECK(a.strides()[1] == 1, "a must be row major");
+  TORCH_CHECK(b.strides()[1] == 1, "b must be column major");
+  TORCH_CHECK(d.scalar_type() == torch::kBFloat16 || d.scalar_type() == torch::kHalf,
+              "dtype must be kFloat16 or kBFloat16");
+  const int64_t num_experts = problem_sizes.size(0);
+  TORCH_CHECK(num_experts >= 1 && num_experts <= ESMOE_MAX_EXPERTS,
+              "Number of experts cannot exceed 1024, the maximum number of threads per block.");
+  // a and b are read through data_ptr() as e4m3 bytes whatever their dtype: the reference's own test
+  // passes 2-byte tensors that the quant op filled with bytes
+  // (test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:72-76,95-101).
+  TORCH_CHECK(a.stride(0) == a.size(1), "a must be packed");
+  TORCH_CHECK(b.size(0) == num_experts && b.stride(2) == b.size(1) && b.stride(0) == b.size(1) * b.size(2),
+              "b must be the column-major (num_experts, k, n) view of a packed (num_experts, n, k) tensor");
+  const int64_t total_rows = a.size(0), k = a.size(1), n = b.size(2);
+  TORCH_CHECK(d.dim() == 2 && d.size(0) == total_rows && d.size(1) == n && d.is_contiguous(),
+              "d must be a contiguous (num_tokens, n) tensor");
+  TORCH_CHECK(sfa.element_size() == 1 && sfb.element_size() == 1, "scale factors must be 1-byte E8M0");
+  TORCH_CHECK(sfb.numel() >= num_experts * n * (k / 32), "sfb is smaller than num_experts * n * k / 32 bytes");
+  TORCH_CHECK(expert_offsets.dtype() == torch::kInt32 && blockscale_offsets.dtype() == torch::kInt32,
+              "offset tensors must be int32");
+  TORCH_CHECK(blockscale_offsets.dim() == 1 && blockscale_offsets.size(0) == num_experts,
+              "blockscale_offsets must be 1D and have size equal to the number of experts");
+  TORCH_CHECK(total_rows < (int64_t(1) << 31), "tensor too large");
+
+  require_device(a, "es_sm100_mxfp8_blockscaled_grouped_mm");
+  for (const torch::Tensor* t :
+       {&b, &sfa, &sfb, (const torch::Tensor*)&d, &problem_sizes, &expert_offsets, &blockscale_offsets}) {
+    TORCH_CHECK(t->device() == a.device(), "all tensors must be on the same device");
+  }
+  TORCH_CHECK(problem_sizes.is_contiguous() && expert_offsets.is_contiguous() && blockscale_offsets.is_contiguous(),
+              "metadata tensors must be contiguous");
+  if (total_rows == 0) return;
+  c10::DeviceGuard guard(a.device());
+  torch::Tensor ws = schedule_scratch(nullptr, num_experts, a);
+  int rc = esmoe_mxfp8_grouped_mm(d.data_ptr(), out_dtype_of(d), a.data_ptr(), b.data_ptr(),
+                                  (const uint8_t*)sfa.data_ptr(), (const uint8_t*)sfb.data_ptr(),
+                                  problem_sizes.data_ptr<int32_t>(), expert_offsets.data_ptr<int32_t>(),
+                                  blockscale_offsets.data_ptr<int32_t>(), (int)num_experts, (int)total_rows, (int)n,
+                                  (int)k, /*force_bm=*/0, ws.data_ptr(), ws.nbytes(), current_stream(a));
+  check_rc(rc, "es_sm100_mxfp8_blockscaled_grouped_mm");
+}
+
+void es_sm100_mxfp8_blockscaled_grouped_quant(const torch::Tensor& input, const torch::Tensor& problem_sizes,
+                                              const torch::Tensor& expert_offsets,
+                                              const torch::Tensor& blockscale_offsets, torch::Tensor& quant_output,
+                                              torch::Tensor& scale_factor) {
+  TORCH_CHECK(input.dim() == 2, "input must be 2D tensor");
+  TORCH_CHECK(input.size(1) % 128 == 0, "k must align to 128");
+  TORCH_CHECK(input.strides()[1] == 1, "input must be row major");
+  TORCH_CHECK(problem_sizes.dim() == 2, "problem_sizes must be 2D tensor");
+  const int64_t groups = problem_sizes.size(0);
+  TORCH_CHECK(expert_offsets.dim() == 1 && expert_offsets.size(0) == groups,
+              "expert_offsets must be 1D and have size equal to the number of groups");
+  TORCH_CHECK(blockscale_offsets.dim() == 1 && blockscale_offsets.size(0) == groups,
+              "blockscale_offsets must be 1D and have size equal to the number of groups");
+  TORCH_CHECK(input.scalar_type() == torch::kBFloat16 || input.scalar_type() == torch::kHalf,
+              "dtype must be kFloat16 or kBFloat16");
+  TORCH_CHECK(problem_sizes.size(1) == 3 && problem_sizes.dtype() == torch::kInt32 &&
+                  expert_offsets.dtype() == torch::kInt32 && blockscale_offsets.dtype() == torch::kInt32,
+              "problem_sizes (groups, 3), expert_offsets and blockscale_offsets must be int32");
+  TORCH_CHECK(groups >= 1 && groups <= ESMOE_MAX_EXPERTS, "number of groups must be in [1, 1024]");
+  TORCH_CHECK(input.stride(0) == input.size(1), "input must be packed");
+  const int64_t total_rows = input.size(0), k = input.size(1);
+  // The reference's test hands over zeros_like(input) (2-byte elements) and lets the kernel write
+  // bytes into it (test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:72); any contiguous
+  // tensor with room for rows*k bytes is accepted.
+  TORCH_CHECK(quant_output.is_contiguous() && (int64_t)quant_output.nbytes() >= total_rows * k,
+              "quant_output must be contiguous and hold at least rows * k bytes");
+  TORCH_CHECK(scale_factor.is_contiguous() && scale_factor.element_size() == 1,
+              "scale_factor must be a contiguous 1-byte tensor");
+  const int64_t sf_rows = (scale_factor.numel() / (k / 32)) / 128 * 128;
+  TORCH_CHECK(total_rows < (int64_t(1) << 31) && sf_rows < (int64_t(1) << 31), "tensor too large");
+
+  require_device(input, "es_sm100_mxfp8_blockscaled_grouped_quant");
+  for (const torch::Tensor* t : {&problem_sizes, &expert_offsets, &blockscale_offsets, (const torch::Tensor*)&quant_output,
+                                 (const torch::Tensor*)&scale_factor}) {
+    TORCH_CHECK(t->device() == input.device(), "all tensors must be on the same device");
+  }
+  TORCH_CHECK(problem_sizes.is_contiguous() && expert_offsets.is_contiguous() && blockscale_offsets.is_contiguous(),
+              "metadata tensors must be contiguous");
+  if (total_rows == 0) return;
+  c10::DeviceGuard guard(input.device());
+  int rc = esmoe_mxfp8_grouped_quant(
+      input.data_ptr(), input.scalar_type() == torch::kBFloat16 ? ESMOE_IN_BF16 : ESMOE_IN_FP16,
+      problem_sizes.data_ptr<int32_t>(), expert_offsets.data_ptr<int32_t>(), blockscale_offsets.data_ptr<int32_t>(),
+      quant_output.data_ptr(), (uint8_t*)scale_factor.data_ptr(), (int)groups, (int)total_rows, (int)sf_rows, (int)k,
+      current_stream(input));
+  check_rc(rc, "es_sm100_mxfp8_blockscaled_grouped_quant");
+}
+
+TORCH_LIBRARY(expert_specialization, m) {
+  m.def(
+      "es_fp8_blockwise_scaled_grouped_mm(Tensor output, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, Tensor "
+      "stride_a, Tensor stride_b, Tensor stride_d, Tensor problem_sizes, Tensor expert_offsets, Tensor workspace) -> "
+      "()");
+  m.def(
+      "es_sm100_mxfp8_blockscaled_grouped_mm(Tensor a, Tensor b, Tensor sfa, Tensor sfb, Tensor d, Tensor "
+      "problem_sizes, Tensor expert_offsets, Tensor blockscale_offsets) -> ()");
+  m.def(
+      "es_sm100_mxfp8_blockscaled_grouped_quant(Tensor input, Tensor problem_sizes, Tensor expert_offsets, Tensor "
+      "blockscale_offsets, Tensor quant_output, Tensor scale_factor) -> () ");
+}
+
+TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
+  m.impl("es_fp8_blockwise_scaled_grouped_mm", &es_fp8_blockwise_scaled_grouped_mm);
+  m.impl("es_sm100_mxfp8_blockscaled_grouped_mm", &es_sm100_mxfp8_blockscaled_grouped_mm);
+  m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
+}
+
+// Same functions on the CPU key: the checks run, then require_device() raises.
+TORCH_LIBRARY_IMPL(expert_specialization, CPU, m) {
+  m.impl("es_fp8_blockwise_scaled_grouped_mm", &es_fp8_blockwise_scaled_grouped_mm);
+  m.impl("es_sm100_mxfp8_blockscaled_grouped_mm", &es_sm100_mxfp8_blockscaled_grouped_mm);
+  m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
+}

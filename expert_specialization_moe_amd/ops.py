@@ -1,0 +1,28 @@
+"""Python entry points with the reference's names and positional orders
+(expert_specialization/ops.py:4-50).  Each forwards to the operator registered
+under ``torch.ops.expert_specialization`` and returns None; results are written
+into the caller's output tensor.
+"""
+import torch
+
+_ns = torch.ops.expert_specialization
+
+
+def es_fp8_blockwise_scaled_grouped_mm(output, a, b, scales_a, scales_b, stride_a, stride_b, stride_d,
+                                       problem_sizes, expert_offsets, workspace):
+    """output[off_e:off_e+M_e] = (scales_a * a)[rows of e] @ (scales_b * b)[e]  (ops.py:4-29)."""
+    _ns.es_fp8_blockwise_scaled_grouped_mm.default(
+        output, a, b, scales_a, scales_b, stride_a, stride_b, stride_d, problem_sizes, expert_offsets, workspace)
+
+
+def es_sm100_mxfp8_blockscaled_grouped_mm(output, a, b, sfa, sfb, problem_sizes, expert_offsets, blockscale_offsets):
+    """MXFP8 grouped GEMM; note the operator takes ``output`` fifth (ops.py:32-37)."""
+    _ns.es_sm100_mxfp8_blockscaled_grouped_mm.default(
+        a, b, sfa, sfb, output, problem_sizes, expert_offsets, blockscale_offsets)
+
+
+def es_sm100_mxfp8_blockscaled_grouped_quant(input, problem_sizes, expert_offsets, blockscale_offsets,
+                                             quant_output, scale_factor):
+    """bf16/fp16 rows -> e4m3 bytes + swizzled E8M0 scales (ops.py:40-50)."""
+    _ns.es_sm100_mxfp8_blockscaled_grouped_quant.default(
+        input, problem_sizes, expert_offsets, blockscale_offsets, quant_output, scale_factor)

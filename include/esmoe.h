@@ -1,0 +1,121 @@
+/*
+ * C ABI of the MI355X (gfx950) expert-specialized grouped-GEMM library (libesmoe.so).
+ *
+ * Plain pointers and sizes only; every pointer is device memory unless stated.
+ * All entry points enqueue work on `stream` (a hipStream_t passed as void*) and
+ * return without synchronising.  Return value: 0 on success, a negative
+ * ESMOE_ERR_* for rejected arguments, a positive hipError_t if a launch failed.
+ * esmoe_last_error() gives a message for the calling thread's last failure.
+ *
+ * Per-expert metadata follows the reference operators exactly:
+ *   problem_sizes     int32 [E,3] rows (M_e, N, K)      (N and K equal for all experts)
+ *   expert_offsets    int32 [E]   first row of expert e in the packed [sum M, .] tensors
+ *   blockscale_offsets int32 [E]  first row of expert e in the swizzled scale tensor
+ *                                 (prefix sum of M_e rounded up to 128)
+ * They are read on the device only; no entry point copies them to the host.
+ */
+#ifndef ESMOE_H_
+#define ESMOE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ESMOE_OUT_BF16 0
+#define ESMOE_OUT_FP16 1
+#define ESMOE_IN_BF16 0
+#define ESMOE_IN_FP16 1
+
+#define ESMOE_ERR_INVALID_ARGUMENT (-1)
+#define ESMOE_ERR_WORKSPACE_TOO_SMALL (-2)
+#define ESMOE_ERR_UNSUPPORTED_DEVICE (-3)
+
+#define ESMOE_MAX_EXPERTS 1024 /* same limit as the reference, es_fp8_blockwise_launcher.cuh:53 */
+
+/* Bytes of device scratch the two GEMM entry points need for `num_experts` experts
+ * (the device-built tile schedule and its work counter). */
+size_t esmoe_gemm_workspace_bytes(int num_experts);
+
+/*
+ * FP8-blockwise scaled grouped GEMM.
+ * Replaces es_fp8_blockwise_scaled_grouped_mm
+ *   (expert_specialization/csrc/cuda/es_fp8_blockwise.cu:34-193, schema
+ *    expert_specialization/csrc/expert_specialization.cpp:57-60).
+ *
+ *   out[off_e + m, n] = cast( sum_kb sa[off_e + m, kb] * sb[e, n/128, kb]
+ *                               * sum_{k in kb} a[off_e + m, k] * b[e, n, k] )
+ *
+ *   out  [total_rows, N] bf16 or fp16 (out_dtype), row-major
+ *   a    [total_rows, K] e4m3fn bytes, row-major
+ *   b    [E, N, K] e4m3fn bytes (the physical layout behind the reference's (E,K,N) view)
+ *   sa   [total_rows, K/128] fp32;  sb [E, N/128, K/128] fp32
+ * N % 128 == 0, K % 128 == 0, 1 <= E <= ESMOE_MAX_EXPERTS.
+ * force_bm: 0 lets the device-side schedule pick an M-tile shape per expert;
+ *           16/32/64/128/256 forces that single shape for every tile (benchmarking).
+ * Rows of `out` that belong to no expert (M_e == 0) are not written.
+ */
+int esmoe_fp8_blockwise_grouped_mm(void* out, int out_dtype, const void* a, const void* b, const float* sa,
+                                   const float* sb, const int32_t* problem_sizes, const int32_t* expert_offsets,
+                                   int num_experts, int total_rows, int n, int k, int force_bm, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+
+/*
+ * MXFP8 block-scaled grouped GEMM (e4m3 data, E8M0 scale per 1x32 block along K).
+ * Replaces es_sm100_mxfp8_blockscaled_grouped_mm
+ *   (expert_specialization/csrc/cuda/es_sm100_mxfp8_blockscaled.cu:5-40, schema
+ *    expert_specialization/csrc/expert_specialization.cpp:61-63).
+ *
+ *   d[off_e + m, n] = cast( sum_k a[off_e+m,k] 2^(sfa-127) * b[e,n,k] 2^(sfb-127) )
+ *
+ *   sfa: swizzled 128x4 scale tiles, expert e at byte blockscale_offsets[e]*(K/32)
+ *   sfb: swizzled 128x4 scale tiles, expert e at byte e*N*(K/32), N rows
+ *   (tile layout: es_sm100_mxfp8_blockscaled_group_quant.cuh:25,294-307)
+ */
+int esmoe_mxfp8_grouped_mm(void* d, int out_dtype, const void* a, const void* b, const uint8_t* sfa,
+                           const uint8_t* sfb, const int32_t* problem_sizes, const int32_t* expert_offsets,
+                           const int32_t* blockscale_offsets, int num_experts, int total_rows, int n, int k,
+                           int force_bm, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * MXFP8 grouped quantisation: bf16/fp16 rows -> e4m3 bytes + swizzled E8M0 scales.
+ * Replaces es_sm100_mxfp8_blockscaled_grouped_quant
+ *   (expert_specialization/csrc/cuda/es_sm100_mxfp8_blockscaled_group_quant.cu:5-39,
+ *    ..._group_quant.cuh:261-405, schema expert_specialization.cpp:64-66).
+ *
+ *   in [total_rows, K] bf16 or fp16 (in_dtype);  q [total_rows, K] bytes;
+ *   sf: `sf_rows` rows of K/32 scale bytes (sf_rows % 128 == 0, >= the largest
+ *       blockscale_offsets[e] + M_e rounded up to 128); expert e's scales start at byte
+ *       blockscale_offsets[e]*(K/32); rows < M_e are defined, padding rows of an expert's
+ *       last 128-row tile are written as 0 (the reference leaves them unspecified).
+ *   blockscale_offsets must be non-decreasing multiples of 128 (the reference's callers
+ *   build them as the prefix sum of M_e rounded up to 128).
+ * Only columns 0 (M_e) and 2 (K) of problem_sizes are used, as in the reference (:281-282).
+ */
+int esmoe_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* problem_sizes,
+                              const int32_t* expert_offsets, const int32_t* blockscale_offsets, void* q,
+                              uint8_t* sf, int num_experts, int total_rows, int sf_rows, int k, void* stream);
+
+/*
+ * Host mirrors of the device-side tile schedule, for inspection and CPU tests; they touch no GPU.
+ * No counterpart in the reference (its schedule lives inside CUTLASS's grouped tile scheduler).
+ * esmoe_host_schedule fills `ws_host` (esmoe_gemm_workspace_bytes(E) bytes of host memory) from host
+ * copies of problem_sizes exactly as the schedule kernel fills the device workspace;
+ * esmoe_host_decode_item maps work item `item` to out5 = {expert, tile rows, tile cols, m0, n0}.
+ */
+int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int32_t* ws_host);
+int esmoe_host_decode_item(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
+                           int force_bm, int item, int32_t* out5);
+
+/* Message describing the calling thread's most recent failure ("" if none). */
+const char* esmoe_last_error(void);
+
+/* Library version string. */
+const char* esmoe_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ESMOE_H_ */
