@@ -145,3 +145,38 @@ def make_fp8_blockwise_operands(prob: Problem, device, seed=0, out_dtype=torch.b
         "output": torch.empty((total, n), dtype=out_dtype, device=device),
         "a_hp": a,
     }
+
+
+def make_mxfp8_operands(prob: Problem, device, seed=0, out_dtype=torch.bfloat16, weight_std=0.02, in_dtype=torch.bfloat16):
+    """Operands of the MXFP8 quant + GEMM pair, built the way the reference's end-to-end test does
+    (test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:42-101): activations and weights are both
+    quantised by the grouped quant op, the weights through the auxiliary problem list [N, M, K] with
+    offsets e*N.  Needs a GPU (it calls the op)."""
+    from . import ops
+
+    e, n, k = prob.num_experts, prob.n, prob.k
+    total = prob.total_rows
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    a = torch.randn((total, k), generator=gen, dtype=torch.float32).to(in_dtype).to(device)
+    w = torch.empty((e * n, k), dtype=in_dtype, device=device)
+    for i in range(e):
+        w[i * n:(i + 1) * n] = (torch.randn((n, k), generator=gen, dtype=torch.float32) * weight_std).to(in_dtype).to(device)
+    ps = torch.tensor([[m, n, k] for m in prob.rows], dtype=torch.int32, device=device)
+    eo = torch.tensor(offsets_of(prob.rows), dtype=torch.int32, device=device)
+    bso_np, sf_rows = blockscale_offsets_of(prob.rows)
+    bso = torch.tensor(bso_np, dtype=torch.int32, device=device)
+    aux_ps = torch.tensor([[n, m, k] for m in prob.rows], dtype=torch.int32, device=device)
+    aux_eo = torch.arange(e, dtype=torch.int32, device=device) * n
+    a_q = torch.zeros((total, k), dtype=torch.float8_e4m3fn, device=device)
+    sfa = torch.zeros((max(sf_rows, 128), k // 32), dtype=torch.uint8, device=device)
+    b_q = torch.zeros((e * n, k), dtype=torch.float8_e4m3fn, device=device)
+    sfb = torch.zeros((e, n, k // 32), dtype=torch.uint8, device=device)
+    ops.es_sm100_mxfp8_blockscaled_grouped_quant(a, ps, eo, bso, a_q, sfa)
+    ops.es_sm100_mxfp8_blockscaled_grouped_quant(w, aux_ps, aux_eo, aux_eo, b_q, sfb)
+    return {
+        "a_hp": a, "w_hp": w, "a": a_q, "b": b_q.view(e, n, k).transpose(1, 2), "b_phys": b_q.view(e, n, k),
+        "sfa": sfa, "sfb": sfb.view(e, n, k // 32).transpose(1, 2), "sfb_phys": sfb,
+        "problem_sizes": ps, "expert_offsets": eo, "blockscale_offsets": bso,
+        "aux_problem_sizes": aux_ps, "aux_expert_offsets": aux_eo,
+        "output": torch.empty((total, n), dtype=out_dtype, device=device),
+    }

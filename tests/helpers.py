@@ -68,3 +68,25 @@ def capi_fp8_mm(native, ops, force_bm=0, out=None):
     assert rc == 0, (rc, native.last_error())
     torch.cuda.synchronize()
     return out
+
+
+def capi_mx_mm(native, ops, force_bm=0, out=None):
+    lib = native.lib
+    out = ops["output"] if out is None else out
+    e = ops["problem_sizes"].size(0)
+    total, k = ops["a"].shape
+    n = ops["b_phys"].size(1)
+    need = lib.esmoe_gemm_workspace_bytes(e)
+    ws = torch.empty((need,), dtype=torch.uint8, device=out.device)
+    rc = lib.esmoe_mxfp8_grouped_mm(
+        ptr(out), 0 if out.dtype == torch.bfloat16 else 1, ptr(ops["a"]), ptr(ops["b_phys"]), ptr(ops["sfa"]),
+        ptr(ops["sfb_phys"]), ptr(ops["problem_sizes"]), ptr(ops["expert_offsets"]), ptr(ops["blockscale_offsets"]),
+        e, total, n, k, force_bm, ptr(ws), need, stream_ptr())
+    assert rc == 0, (rc, native.last_error())
+    torch.cuda.synchronize()
+    return out
+
+
+def hp_to_f32(t: torch.Tensor) -> np.ndarray:
+    """bf16/fp16 tensor -> float32 numpy (exact)."""
+    return t.detach().float().cpu().numpy()
