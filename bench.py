@@ -1,0 +1,177 @@
+#!/usr/bin/env python3
+"""Benchmark of the expert-specialized grouped GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4] [--force-bm 0|16|...]
+
+One "step" is one call of the operator (through torch.ops.expert_specialization.*) over one batch
+of synthetic, already-quantised operands resident in HBM.  Prints ONE JSON line.  The default
+workload is c1: the DeepSeek-V3 gate_up projection, one GPU's 32-expert share (K=7168, N=4096,
+FP8-blockwise, 4096 tokens routed top-8 over 256 experts with Zipf(1.2) popularity, seed 0).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c1", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--tokens", type=int, default=8192, help="c3 only")
+    ap.add_argument("--routing", default="zipf", choices=["zipf", "uniform"], help="c3 only")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--force-bm", type=int, default=0, help="single M-tile shape for every expert (0 = device schedule)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline sample")
+    return ap.parse_args()
+
+
+def cpu_baseline(prob, ops, budget_s):
+    """The oracle's dequantise + fp32 matmul (the reference's torch CPU path) timed on this host on a
+    bounded sample: experts in index order until the time budget is used."""
+    from oracle import fp8_blockwise as ofp8
+    from oracle import mxfp8 as omx
+    import numpy as np
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    cores = torch.get_num_threads()
+    rows = prob.rows
+    offs = [0]
+    for m in rows[:-1]:
+        offs.append(offs[-1] + m)
+    flops = 0.0
+    used = 0.0
+    done = 0
+    a_codes = ops["a"].contiguous().view(torch.uint8).cpu().numpy()
+    for e, m in enumerate(rows):
+        if m == 0:
+            done += 1
+            continue
+        b_e = ops["b_phys"][e:e + 1].contiguous().view(torch.uint8).cpu().numpy()
+        ps = [[m, prob.n, prob.k]]
+        if prob.kind == "fp8_blockwise":
+            sa = ops["scales_a"][offs[e]:offs[e] + m].float().cpu().numpy()
+            sb = ops["scales_b_phys"][e:e + 1].float().cpu().numpy()
+            t0 = time.perf_counter()
+            ofp8.grouped_mm(a_codes[offs[e]:offs[e] + m], b_e, sa, sb, ps, [0])
+            used += time.perf_counter() - t0
+        else:
+            bso = int(ops["blockscale_offsets"][e])
+            kc = prob.k // 32
+            sfa = ops["sfa"].reshape(-1)[bso * kc:(bso + (m + 127) // 128 * 128) * kc].cpu().numpy()
+            sfb = ops["sfb_phys"][e].reshape(-1).cpu().numpy()
+            t0 = time.perf_counter()
+            omx.grouped_mm(a_codes[offs[e]:offs[e] + m], b_e, sfa, sfb, ps, [0], [0])
+            used += time.perf_counter() - t0
+        flops += 2.0 * m * prob.n * prob.k
+        done += 1
+        if used > budget_s:
+            break
+    return {
+        "value": flops / used / 1e12 if used else 0.0, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"first {done} of {len(rows)} experts of the same workload ({flops / 1e9:.1f} GFLOP, {used:.1f} s)",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    import expert_specialization_moe_amd as es
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import workloads as W
+
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    prob = W.config_problem(args.config, seed=args.seed, tokens=args.tokens, routing=args.routing)
+    mx = prob.kind == "mxfp8"
+    ops = (W.make_mxfp8_operands if mx else W.make_fp8_blockwise_operands)(prob, dev, seed=args.seed)
+    lib = _native.lib
+    e, n, k, total = prob.num_experts, prob.n, prob.k, prob.total_rows
+    ws_bytes = lib.esmoe_gemm_workspace_bytes(e)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+    import ctypes
+
+    def vp(t):
+        return ctypes.c_void_p(t.data_ptr())
+
+    if args.force_bm:
+        # single-tile-shape baseline: same kernel, one M-tile height for every expert (C ABI only)
+        def step():
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            if mx:
+                rc = lib.esmoe_mxfp8_grouped_mm(vp(ops["output"]), 0, vp(ops["a"]), vp(ops["b_phys"]), vp(ops["sfa"]),
+                                                vp(ops["sfb_phys"]), vp(ops["problem_sizes"]), vp(ops["expert_offsets"]),
+                                                vp(ops["blockscale_offsets"]), e, total, n, k, args.force_bm, vp(ws),
+                                                ws_bytes, stream)
+            else:
+                rc = lib.esmoe_fp8_blockwise_grouped_mm(vp(ops["output"]), 0, vp(ops["a"]), vp(ops["b_phys"]),
+                                                        vp(ops["scales_a"]), vp(ops["scales_b_phys"]),
+                                                        vp(ops["problem_sizes"]), vp(ops["expert_offsets"]), e, total, n,
+                                                        k, args.force_bm, vp(ws), ws_bytes, stream)
+            assert rc == 0, _native.last_error()
+    elif mx:
+        def step():
+            es.es_sm100_mxfp8_blockscaled_grouped_mm(ops["output"], ops["a"], ops["b"], ops["sfa"], ops["sfb"],
+                                                     ops["problem_sizes"], ops["expert_offsets"],
+                                                     ops["blockscale_offsets"])
+    else:
+        def step():
+            es.es_fp8_blockwise_scaled_grouped_mm(ops["output"], ops["a"], ops["b"], ops["scales_a"], ops["scales_b"],
+                                                  ops["stride_a"], ops["stride_b"], ops["stride_d"],
+                                                  ops["problem_sizes"], ops["expert_offsets"], ops["workspace"])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = start.elapsed_time(stop) / args.steps
+
+    flops = W.gemm_flops(prob.rows, n, k)
+    nbytes = W.gemm_bytes(prob.rows, n, k, prob.kind)
+    t_roof = W.gemm_roofline_seconds(prob.rows, n, k, prob.kind)
+    t = ms_per_step * 1e-3
+    hbm_bound = nbytes / W.HBM_BYTES_PER_S >= flops / W.FP8_FLOPS_PER_S
+    if hbm_bound:
+        roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": W.HBM_BYTES_PER_S / 1e9, "unit": "GB/s"}
+    else:
+        roof = {"bound": "mfma", "achieved": flops / t / 1e12, "peak": W.FP8_FLOPS_PER_S / 1e12, "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["algorithmic_bytes"] = nbytes
+    roof["roofline_us"] = t_roof * 1e6
+    out = {
+        "metric": "useful FP8 TFLOP/s + % of roofline, DSv3-shape grouped GEMM, Zipf routing",
+        "value": flops / t / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 (fp32 accumulate, bf16 out)", "data": "synthetic",
+        "config": {"workload": f"{prob.name}: E={e} K={k} N={n} rows={total} max_rows={max(prob.rows)} "
+                               f"active={sum(1 for m in prob.rows if m)} kind={prob.kind} seed={args.seed}",
+                   "force_bm": args.force_bm, "routing_meta": prob.meta},
+        "roofline": roof, "wall_ms_per_step": wall * 1e3 / args.steps,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(prob, ops, args.cpu_seconds)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -286,7 +286,7 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
   ESMOE_CASE(16, 2)
 #endif
 #ifndef ESMOE_WAVES_PER_SIMD
-#define ESMOE_WAVES_PER_SIMD 2
+#define ESMOE_WAVES_PER_SIMD 1
 #endif
 
 template <bool MX>

@@ -123,14 +123,15 @@ def make_fp8_blockwise_operands(prob: Problem, device, seed=0, out_dtype=torch.b
     """Operands of es_fp8_blockwise_scaled_grouped_mm in the layouts the reference's callers build
     (test/test_es_grouped_gemm.py:143-179).  Returns a dict of tensors on `device`."""
     e, n, k = prob.num_experts, prob.n, prob.k
-    gen = torch.Generator(device="cpu").manual_seed(seed)
+    gdev = device if torch.device(device).type == "cuda" else "cpu"   # values are seeded per device type
+    gen = torch.Generator(device=gdev).manual_seed(seed)
     total = prob.total_rows
-    a = torch.randn((total, k), generator=gen, dtype=torch.float32).to(torch.bfloat16).to(device)
+    a = torch.randn((total, k), generator=gen, dtype=torch.float32, device=gdev).to(torch.bfloat16).to(device)
     a_q, sa = quant_act_1x128(a)
     b_q = torch.empty((e, n, k), dtype=torch.float8_e4m3fn, device=device)
     sb = torch.empty((e, n // 128, k // 128), dtype=torch.float32, device=device)
     for i in range(e):
-        w = (torch.randn((n, k), generator=gen, dtype=torch.float32) * weight_std).to(device)
+        w = (torch.randn((n, k), generator=gen, dtype=torch.float32, device=gdev) * weight_std).to(device)
         b_q[i], sb[i] = quant_weight_128x128(w)
     ps = torch.tensor([[m, n, k] for m in prob.rows], dtype=torch.int32, device=device)
     eo = torch.tensor(offsets_of(prob.rows), dtype=torch.int32, device=device)
@@ -156,11 +157,12 @@ def make_mxfp8_operands(prob: Problem, device, seed=0, out_dtype=torch.bfloat16,
 
     e, n, k = prob.num_experts, prob.n, prob.k
     total = prob.total_rows
-    gen = torch.Generator(device="cpu").manual_seed(seed)
-    a = torch.randn((total, k), generator=gen, dtype=torch.float32).to(in_dtype).to(device)
+    gdev = device if torch.device(device).type == "cuda" else "cpu"
+    gen = torch.Generator(device=gdev).manual_seed(seed)
+    a = torch.randn((total, k), generator=gen, dtype=torch.float32, device=gdev).to(in_dtype).to(device)
     w = torch.empty((e * n, k), dtype=in_dtype, device=device)
     for i in range(e):
-        w[i * n:(i + 1) * n] = (torch.randn((n, k), generator=gen, dtype=torch.float32) * weight_std).to(in_dtype).to(device)
+        w[i * n:(i + 1) * n] = (torch.randn((n, k), generator=gen, dtype=torch.float32, device=gdev) * weight_std).to(in_dtype)
     ps = torch.tensor([[m, n, k] for m in prob.rows], dtype=torch.int32, device=device)
     eo = torch.tensor(offsets_of(prob.rows), dtype=torch.int32, device=device)
     bso_np, sf_rows = blockscale_offsets_of(prob.rows)
