@@ -29,6 +29,8 @@ HIP_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-mcode-object-version=5",
     # packed fp32 VALU ops are kept out of the device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results go to VGPRs: the fp32 scale-and-accumulate of the FP8-blockwise path reads them with VALU ops
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument",
     f"-I{INCLUDE}", f"-I{CSRC}",
 ]

@@ -68,12 +68,7 @@ esmoe::SchedPolicy make_policy(int force_bm) {
   esmoe::SchedPolicy p;
   p.force_mt = force_bm / 16;
   p.big_mt = env_int("ESMOE_BIG_MT", 8);
-  p.nt_light = env_int("ESMOE_NT_LIGHT", 4);
-  p.nt_heavy = env_int("ESMOE_NT_HEAVY", 4);
-  p.light_max_mt = env_int("ESMOE_LIGHT_MAX_MT", 4);
   p.order = env_int("ESMOE_ORDER", 0);
-  if (p.force_mt == 16 || p.big_mt == 16) p.nt_heavy = 2;  // the 256-row tile exists 128 columns wide only
-  if (p.force_mt && p.force_mt > p.light_max_mt && p.force_mt < 16 && p.nt_heavy == 1) p.nt_heavy = 2;
   return p;
 }
 

@@ -3,8 +3,18 @@
 // One launch serves every expert.  A one-workgroup schedule kernel turns
 // problem_sizes into a list of workgroup tiles (schedule.h); persistent workgroups
 // then pull tiles from an atomic counter.  A workgroup is 4 wavefronts laid out
-// along N; a tile is (MT*16) rows x (NT*64) columns and each wavefront owns
-// NT*16 columns of it.
+// along N; a tile is (MT*16) token rows x (NT*64) weight rows and each wavefront
+// owns NT*16 weight rows of it.
+//
+// Data movement.  Per 128-wide K block the workgroup loads the token rows and the
+// weight rows of its tile with lane-contiguous 16-byte loads (8 lanes cover one
+// 128-byte row segment, so the texture-address unit sees whole cache lines), keeps
+// them in registers for S-1 K blocks (the global prefetch distance) and then writes
+// them to a double-buffered LDS tile with 144-byte row pitch.  MFMA operand
+// fragments are read back from LDS (16 bytes per lane, conflict-free down a column
+// of rows).  Loading fragments straight from global memory is ~4x slower per CU:
+// a fragment puts consecutive lanes on different rows, i.e. 64 separate 16-byte
+// requests per instruction.
 //
 // MFMA mapping (v_mfma[_scale]_f32_16x16x128_f8f6f4, both operands e4m3):
 //   * the weight rows ride on the instruction's "A" side and the token rows on its
@@ -14,9 +24,6 @@
 //     [16*(l/16), +16) and [64 + 16*(l/16), +16) of the 128-wide K block;
 //   * for the scaled form lane l supplies the E8M0 scale of row (l % 16),
 //     K sub-block (l / 16) in byte 0 of the scale register.
-// Weights stream from global memory straight into registers (each wavefront owns
-// its rows, nothing to share); token rows are shared by the 4 wavefronts and are
-// staged through double-buffered LDS.
 //
 // FP8-blockwise arithmetic follows the reference's blockwise mainloop order
 // (es_fp8_blockwise_traits.cuh:35,60): each 128-wide K block is multiplied into a
@@ -37,8 +44,6 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int kLdsRow = 144;  // 128 data bytes + 16 pad: conflict-free 16-byte reads down a column of rows
-constexpr int kMaxMT = 16;
-constexpr int kLdsBuf = kMaxMT * 16 * kLdsRow;
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   v8i r;
@@ -47,20 +52,47 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   return r;
 }
 
+// LDS layout of one K-block buffer of a tile: token rows, weight rows, then the block's scales.
 template <int MT, int NT, bool MX>
-struct TileRegs {
-  v4i w[NT][2];       // weight fragments of one K block
-  float sa[MX ? 1 : MT];  // activation scales of this lane's token row per row tile (fp8-blockwise)
-  float sb;               // weight block scale (fp8-blockwise)
-  int sfw[MX ? NT : 1];   // E8M0 weight scale, already shifted into byte 0 (mxfp8)
-  int sfa[MX ? MT : 1];   // E8M0 activation scale (mxfp8)
+struct TileGeom {
+  static constexpr int BM = MT * 16;
+  static constexpr int BN = NT * 64;
+  static constexpr int kAChunks = BM * 8;   // 16-byte chunks of the token rows of one K block
+  static constexpr int kWChunks = BN * 8;
+  static constexpr int kAPass = (kAChunks + kThreads - 1) / kThreads;
+  static constexpr int kWPass = kWChunks / kThreads;
+  static constexpr int kABytes = BM * kLdsRow;
+  static constexpr int kWBytes = BN * kLdsRow;
+  // scales: fp8-blockwise -> BM floats (sa of the block); mxfp8 -> verbatim 512-byte swizzled tiles,
+  // weight rows first (BN/128 tiles), then token rows (ceil(BM/128) tiles)
+  static constexpr int kSfwChunks = MX ? BN / 4 : 0;
+  static constexpr int kSfaChunks = MX ? ((BM + 127) / 128) * 32 : 0;
+  // every thread stages one scale item (threads past the tile's needs duplicate a valid one), so the
+  // region is sized for 256 items and the pipeline stays free of divergent branches
+  static constexpr int kScaleBytes = MX ? kThreads * 16 : kThreads * 4;
+  static constexpr int kBufBytes = kABytes + kWBytes + ((kScaleBytes + 15) & ~15);
+  static_assert(kWChunks % kThreads == 0, "weight tile must fill whole passes");
+  static_assert(kSfwChunks + kSfaChunks <= kThreads, "one scale chunk per thread");
 };
 
+// Largest LDS footprint over the compiled shapes (two buffers).
+constexpr int kLdsBytes = 2 * ((128 + 256) * kLdsRow + 4096);
+
+// One K block of a tile in flight between global memory and LDS.
 template <int MT, int NT, bool MX>
+struct TileStage {
+  using G = TileGeom<MT, NT, MX>;
+  v4i a[G::kAPass];
+  v4i w[G::kWPass];
+  float sa;   // fp8-blockwise: sa[row of this thread][kb] (threads < BM)
+  float sb;   // fp8-blockwise: sb[e][n-block of this wavefront][kb]
+  v4i sf;     // mxfp8: this thread's 16-byte chunk of the swizzled scale tiles
+};
+
+template <int MT, int NT, bool MX, int S>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds) {
-  constexpr int BM = MT * 16;
-  constexpr int kChunks = BM * 8;  // 16-byte chunks of one K block of the token tile
-  constexpr int APASS = (kChunks + kThreads - 1) / kThreads;
+  using G = TileGeom<MT, NT, MX>;
+  static_assert(2 * G::kBufBytes <= kLdsBytes, "LDS budget");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -68,47 +100,58 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   const int gq = lane >> 4;
   const int K = g.k, N = g.n, KB = K >> 7;
   const long row_base = g.expert_offsets[e];
-
   const int nw0 = n0 + wave * (NT * 16);
   const bool wave_active = nw0 < N;
-  // weight rows of this lane: nw0 + nt*16 + r  (clamped to stay in bounds for idle wavefronts)
-  const int nrow0 = wave_active ? nw0 + r : r;
-  const uint8_t* wbase = (const uint8_t*)g.b + ((long)e * N + nrow0) * K + gq * 16;
-  const long wstep = 16L * K;
 
-  // token-tile staging: chunk c -> row c/8, 16-byte column c%8
-  const uint8_t* asrc[APASS];
-  int adst[APASS];
+  // staging map: chunk c -> row c/8, 16-byte column c%8 (8 consecutive lanes = one 128-byte row
+  // segment).  Addresses are a wave-uniform 64-bit base plus one 32-bit offset per pass.
+  const int srow = tid >> 3, scol = tid & 7;       // pass p handles tile row srow + 32*p
+  const uint8_t* a_base = (const uint8_t*)g.a + (row_base + m0) * K;
+  const uint8_t* w_base = (const uint8_t*)g.b + ((long)e * N + n0) * K;
+  // (a token tile shorter than 32 rows is staged twice by the two halves of the workgroup: same
+  // bytes to the same place, which keeps every thread on the same instruction stream)
+  const int arow0 = srow & (G::BM < 32 ? G::BM - 1 : 31);
+  uint32_t aoff[G::kAPass];
 #pragma unroll
-  for (int p = 0; p < APASS; p++) {
-    int c = tid + p * kThreads;
-    int arow = c >> 3, acol = c & 7;
-    int grow = m0 + arow;
-    if (grow > M - 1) grow = M - 1;
-    asrc[p] = (const uint8_t*)g.a + (row_base + grow) * K + acol * 16;
-    adst[p] = arow * kLdsRow + acol * 16;
+  for (int p = 0; p < G::kAPass; p++) {
+    int row = arow0 + 32 * p;
+    if (row > M - 1 - m0) row = M - 1 - m0;
+    aoff[p] = (uint32_t)row * (uint32_t)K + scol * 16;
   }
-  const int frag_off = r * kLdsRow + gq * 16;
-
-  // per-lane token rows for the scales
-  long srow[MT];
+  uint32_t woff[G::kWPass];
 #pragma unroll
-  for (int mt = 0; mt < MT; mt++) {
-    int grow = m0 + mt * 16 + r;
-    if (grow > M - 1) grow = M - 1;
-    srow[mt] = grow;
+  for (int p = 0; p < G::kWPass; p++) {
+    int row = srow + 32 * p;
+    if (row > N - 1 - n0) row = N - 1 - n0;
+    woff[p] = (uint32_t)row * (uint32_t)K + scol * 16;
   }
-  const float* sa_base = nullptr;
-  const float* sb_base = nullptr;
-  const uint8_t* sfa_base = nullptr;
-  const uint8_t* sfw_base = nullptr;
+  const int sdst = srow * kLdsRow + scol * 16;     // LDS offset of pass 0; pass p adds 32 rows
+  const int adst = arow0 * kLdsRow + scol * 16;
+  constexpr int kScaleOff = G::kABytes + G::kWBytes;
+  const float* sa_src = nullptr;
+  const float* sb_src = nullptr;
+  const uint8_t* sf_src = nullptr;
   if constexpr (!MX) {
-    sa_base = g.sa + row_base * KB;
-    sb_base = g.sb + ((long)e * (N >> 7) + ((wave_active ? nw0 : 0) >> 7)) * KB;
+    int grow = m0 + tid;
+    if (grow > M - 1) grow = M - 1;
+    sa_src = g.sa + (row_base + grow) * KB;
+    sb_src = g.sb + ((long)e * (N >> 7) + ((wave_active ? nw0 : 0) >> 7)) * KB;
   } else {
-    sfa_base = g.sfa + (long)g.blockscale_offsets[e] * (K >> 5);
-    sfw_base = g.sfb + (long)e * N * (K >> 5);
+    const int kc = K >> 5;
+    if (tid < G::kSfwChunks) {
+      int blk = (n0 >> 7) + (tid >> 5);
+      if (blk * 128 >= N) blk = n0 >> 7;
+      sf_src = g.sfb + (long)e * N * kc + (long)blk * KB * 512 + (tid & 31) * 16;
+    } else {
+      int j = tid - G::kSfwChunks;
+      int blk = (m0 >> 7) + (j >> 5);
+      if (j >= G::kSfaChunks || blk * 128 >= M) blk = m0 >> 7;
+      sf_src = g.sfa + (long)g.blockscale_offsets[e] * kc + (long)blk * KB * 512 + (j & 31) * 16;
+    }
   }
+
+  const int frag_off = r * kLdsRow + gq * 16;
+  const int wfrag_off = G::kABytes + wave * (NT * 16) * kLdsRow + frag_off;
 
   v4f acc[NT][MT];
 #pragma unroll
@@ -116,101 +159,122 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  TileRegs<MT, NT, MX> cur, nxt;
-  v4i astage[APASS];
+  TileStage<MT, NT, MX> st[S];
 
-  auto load_regs = [&](TileRegs<MT, NT, MX>& t, int kb) {
-    const uint8_t* wp = wbase + (long)kb * 128;
+  auto load = [&](TileStage<MT, NT, MX>& t, int kb) {
+    const uint8_t* ab = a_base + (long)kb * 128;
+    const uint8_t* wb = w_base + (long)kb * 128;
+#pragma unroll
+    for (int p = 0; p < G::kAPass; p++) {
+      t.a[p] = *(const v4i*)(ab + aoff[p]);
+    }
+#pragma unroll
+    for (int p = 0; p < G::kWPass; p++) t.w[p] = *(const v4i*)(wb + woff[p]);
+    if constexpr (!MX) {
+      t.sa = sa_src[kb];
+      t.sb = sb_src[kb];
+    } else {
+      t.sf = *(const v4i*)(sf_src + (long)kb * 512);
+    }
+  };
+  auto store = [&](const TileStage<MT, NT, MX>& t, int buf) {
+    uint8_t* lb = lds + buf * G::kBufBytes;
+#pragma unroll
+    for (int p = 0; p < G::kAPass; p++) *(v4i*)(lb + adst + p * 32 * kLdsRow) = t.a[p];
+#pragma unroll
+    for (int p = 0; p < G::kWPass; p++) *(v4i*)(lb + sdst + G::kABytes + p * 32 * kLdsRow) = t.w[p];
+    if constexpr (!MX) {
+      *(float*)(lb + kScaleOff + tid * 4) = t.sa;
+    } else {
+      *(v4i*)(lb + kScaleOff + tid * 16) = t.sf;
+    }
+  };
+  auto compute = [&](const TileStage<MT, NT, MX>& t, int buf) {
+    const uint8_t* lb = lds + buf * G::kBufBytes;
+    v8i wf[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
-      t.w[nt][0] = __builtin_nontemporal_load((const v4i*)(wp + nt * wstep));
-      t.w[nt][1] = __builtin_nontemporal_load((const v4i*)(wp + nt * wstep + 64));
+      wf[nt] = join(*(const v4i*)(lb + wfrag_off + nt * 16 * kLdsRow), *(const v4i*)(lb + wfrag_off + nt * 16 * kLdsRow + 64));
     }
-    if constexpr (!MX) {
-#pragma unroll
-      for (int mt = 0; mt < MT; mt++) t.sa[mt] = sa_base[srow[mt] * KB + kb];
-      t.sb = sb_base[kb];
-    } else {
+    int sfw[MX ? NT : 1];
+    if constexpr (MX) {
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        int n = nrow0 + nt * 16;
-        long off = ((long)(n >> 7) * KB + kb) * 512 + (n & 31) * 16 + ((n & 127) >> 5) * 4;
-        t.sfw[nt] = (int)((*(const uint32_t*)(sfw_base + off)) >> (gq * 8));
-      }
-#pragma unroll
-      for (int mt = 0; mt < MT; mt++) {
-        long m = srow[mt];
-        long off = ((m >> 7) * KB + kb) * 512 + (m & 31) * 16 + ((m & 127) >> 5) * 4;
-        t.sfa[mt] = (int)((*(const uint32_t*)(sfa_base + off)) >> (gq * 8));
+        int nl = wave * (NT * 16) + nt * 16 + r;  // weight row inside the tile
+        uint32_t d = *(const uint32_t*)(lb + kScaleOff + (nl >> 7) * 512 + (nl & 31) * 16 + ((nl & 127) >> 5) * 4);
+        sfw[nt] = (int)(d >> (gq * 8));
       }
     }
-  };
-  auto load_a = [&](int kb) {
-#pragma unroll
-    for (int p = 0; p < APASS; p++) {
-      if (APASS * kThreads == kChunks || tid + p * kThreads < kChunks) astage[p] = *(const v4i*)(asrc[p] + (long)kb * 128);
-    }
-  };
-  auto store_a = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < APASS; p++) {
-      if (APASS * kThreads == kChunks || tid + p * kThreads < kChunks) *(v4i*)(lds + buf * kLdsBuf + adst[p]) = astage[p];
-    }
-  };
-  auto compute = [&](const TileRegs<MT, NT, MX>& t, int buf) {
-    const uint8_t* lb = lds + buf * kLdsBuf + frag_off;
+    v4i af[2][2];
+    af[0][0] = *(const v4i*)(lb + frag_off);
+    af[0][1] = *(const v4i*)(lb + frag_off + 64);
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
-      v4i lo = *(const v4i*)(lb + mt * 16 * kLdsRow);
-      v4i hi = *(const v4i*)(lb + mt * 16 * kLdsRow + 64);
-      v8i af = join(lo, hi);
+      if (mt + 1 < MT) {
+        af[(mt + 1) & 1][0] = *(const v4i*)(lb + frag_off + (mt + 1) * 16 * kLdsRow);
+        af[(mt + 1) & 1][1] = *(const v4i*)(lb + frag_off + (mt + 1) * 16 * kLdsRow + 64);
+      }
+      v8i afr = join(af[mt & 1][0], af[mt & 1][1]);
       if constexpr (!MX) {
-        float s = t.sa[mt] * t.sb;
+        float sc = *(const float*)(lb + kScaleOff + (mt * 16 + r) * 4) * t.sb;
         v4f tmp[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
-          tmp[nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(join(t.w[nt][0], t.w[nt][1]), af,
-                                                                       v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+          tmp[nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], afr, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
         }
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
 #pragma unroll
-          for (int i = 0; i < 4; i++) acc[nt][mt][i] = __builtin_fmaf(tmp[nt][i], s, acc[nt][mt][i]);
+          for (int i = 0; i < 4; i++) acc[nt][mt][i] = __builtin_fmaf(tmp[nt][i], sc, acc[nt][mt][i]);
         }
       } else {
+        int ml = (m0 & 127) + mt * 16 + r;  // token row inside its 128-row scale tile(s)
+        uint32_t d = *(const uint32_t*)(lb + kScaleOff + G::kSfwChunks * 16 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4);
+        int sfa = (int)(d >> (gq * 8));
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(join(t.w[nt][0], t.w[nt][1]), af, acc[nt][mt],
-                                                                           0, 0, 0, t.sfw[nt], 0, t.sfa[mt]);
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], afr, acc[nt][mt], 0, 0, 0, sfw[nt], 0, sfa);
         }
       }
     }
   };
 
-  // prologue
-  load_regs(cur, 0);
-  load_a(0);
-  store_a(0);
+  // prologue: S-1 K blocks in flight, the first one into LDS buffer 0
+#pragma unroll
+  for (int j = 0; j < S - 1; j++) {
+    if (j < KB) load(st[j], j);
+  }
+  store(st[0], 0);
   __syncthreads();
 
-  int kb = 0;
-  for (; kb + 2 <= KB; kb += 2) {
-    load_regs(nxt, kb + 1);
-    load_a(kb + 1);
-    if (wave_active) compute(cur, 0);
-    store_a(1);
-    __syncthreads();
-    if (kb + 2 < KB) {
-      load_regs(cur, kb + 2);
-      load_a(kb + 2);
+  // steady state: branch-free so that the outstanding-load counts stay exact
+  int kb0 = 0;
+  for (; kb0 + 2 * S - 2 < KB; kb0 += S) {
+#pragma unroll
+    for (int j = 0; j < S; j++) {
+      const int kb = kb0 + j;
+      load(st[(j + S - 1) % S], kb + S - 1);
+      __builtin_amdgcn_sched_barrier(0);  // keep the phases in program order: the scheduler would
+      compute(st[j], kb & 1);             // otherwise overlap all stages' live ranges and spill
+      __builtin_amdgcn_sched_barrier(0);
+      store(st[(j + 1) % S], (kb + 1) & 1);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (wave_active) compute(nxt, 1);
-    if (kb + 2 < KB) store_a(0);
-    __syncthreads();
   }
-  if (kb < KB) {  // odd number of K blocks: the last one is in `cur` / buffer 0
-    if (wave_active) compute(cur, 0);
-    __syncthreads();
+  // drain: at most 2S-2 K blocks left
+#pragma unroll
+  for (int t = 0; t < 2; t++) {
+#pragma unroll
+    for (int j = 0; j < S; j++) {
+      const int kb = kb0 + t * S + j;
+      if (kb < KB) {
+        if (kb + S - 1 < KB) load(st[(j + S - 1) % S], kb + S - 1);
+        compute(st[j], kb & 1);
+        if (kb + 1 < KB) store(st[(j + 1) % S], (kb + 1) & 1);
+        __syncthreads();
+      }
+    }
   }
 
   // epilogue: lane holds columns nw0 + nt*16 + 4*gq + [0,4) of token row m0 + mt*16 + r
@@ -224,11 +288,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
         for (int nt = 0; nt < NT; nt++) {
           int n = nw0 + nt * 16 + gq * 4;
           if (g.out_dtype == 0) {
-            bf16x4 v = __builtin_convertvector(acc[nt][mt], bf16x4);
-            *(bf16x4*)((__bf16*)g.out + orow + n) = v;
+            *(bf16x4*)((__bf16*)g.out + orow + n) = __builtin_convertvector(acc[nt][mt], bf16x4);
           } else {
-            f16x4 v = __builtin_convertvector(acc[nt][mt], f16x4);
-            *(f16x4*)((_Float16*)g.out + orow + n) = v;
+            *(f16x4*)((_Float16*)g.out + orow + n) = __builtin_convertvector(acc[nt][mt], f16x4);
           }
         }
       }
@@ -278,12 +340,11 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 
 // (MT, NT) tile shapes compiled into the persistent kernel.
 #ifndef ESMOE_VARIANTS
-#define ESMOE_VARIANTS                                 \
-  ESMOE_CASE(1, 1) ESMOE_CASE(1, 2) ESMOE_CASE(1, 4)   \
-  ESMOE_CASE(2, 1) ESMOE_CASE(2, 2) ESMOE_CASE(2, 4)   \
-  ESMOE_CASE(4, 1) ESMOE_CASE(4, 2) ESMOE_CASE(4, 4)   \
-  ESMOE_CASE(8, 2) ESMOE_CASE(8, 4)                    \
-  ESMOE_CASE(16, 2)
+#define ESMOE_VARIANTS \
+  ESMOE_CASE(1, 4) ESMOE_CASE(2, 4) ESMOE_CASE(4, 4) ESMOE_CASE(8, 4) ESMOE_CASE(16, 2)
+#endif
+#ifndef ESMOE_STAGES
+#define ESMOE_STAGES 3
 #endif
 #ifndef ESMOE_WAVES_PER_SIMD
 #define ESMOE_WAVES_PER_SIMD 1
@@ -291,7 +352,7 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 
 template <bool MX>
 __global__ void __launch_bounds__(kThreads, ESMOE_WAVES_PER_SIMD) grouped_gemm_kernel(GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kLdsBuf];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
   __shared__ int s_item;
   int* ws = g.ws;
   const int total = ws[kWsTotal];
@@ -300,7 +361,7 @@ __global__ void __launch_bounds__(kThreads, ESMOE_WAVES_PER_SIMD) grouped_gemm_k
   for (;;) {
     if (threadIdx.x == 0) s_item = atomicAdd(&ws[kWsCounter], 1);
     __syncthreads();
-    const int item = s_item;
+    const int item = __builtin_amdgcn_readfirstlane(s_item);
     __syncthreads();
     if (item >= total) break;
     // position p with item_start[p] <= item < item_start[p+1]
@@ -314,7 +375,7 @@ __global__ void __launch_bounds__(kThreads, ESMOE_WAVES_PER_SIMD) grouped_gemm_k
     const TileCoord t = sched_decode(item - item_start[lo], M, g.n, g.policy);
     const int key = t.mt * 8 + t.nt;
 #define ESMOE_CASE(MT_, NT_) \
-  case (MT_) * 8 + (NT_): gemm_tile<MT_, NT_, MX>(g, e, M, t.m0, t.n0, lds); break;
+  case (MT_) * 8 + (NT_): gemm_tile<MT_, NT_, MX, ((MT_) >= 16 ? 2 : ESMOE_STAGES)>(g, e, M, t.m0, t.n0, lds); break;
     switch (key) {
       ESMOE_VARIANTS
       default: break;

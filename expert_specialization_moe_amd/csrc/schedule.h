@@ -26,9 +26,6 @@ namespace esmoe {
 struct SchedPolicy {
   int force_mt;   // 0 = choose per expert; else every tile uses this MT
   int big_mt;     // MT of the full tiles of a many-row expert (8 or 16)
-  int nt_light;   // NT for tiles with MT <= light_max_mt
-  int nt_heavy;   // NT for taller tiles
-  int light_max_mt;
   int order;      // 0: experts sorted by rows, most rows first; 1: expert index order
 };
 
@@ -45,13 +42,8 @@ ESMOE_HD int sched_cover_mt(int rows, int max_mt) {
   return mt;
 }
 
-// Compiled shapes: MT in {1,2,4} with NT in {1,2,4}; MT = 8 with NT in {2,4}; MT = 16 with NT = 2.
-ESMOE_HD int sched_nt_for(int mt, const SchedPolicy& p) {
-  if (mt >= 16) return 2;
-  int nt = mt <= p.light_max_mt ? p.nt_light : p.nt_heavy;
-  if (mt >= 8 && nt < 2) nt = 2;
-  return nt;
-}
+// Compiled shapes: MT in {1, 2, 4, 8} are 256 columns wide (NT = 4), MT = 16 is 128 wide (NT = 2).
+ESMOE_HD int sched_nt_for(int mt, const SchedPolicy&) { return mt >= 16 ? 2 : 4; }
 
 ESMOE_HD int sched_ntiles(int n, int nt) { return (n + nt * 64 - 1) / (nt * 64); }
 
