@@ -79,6 +79,7 @@ int check_common(const void* out, const void* a, const void* b, const int32_t* p
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "num_experts must be in [1, %d], got %d", ESMOE_MAX_EXPERTS, num_experts);
   if (n <= 0 || n % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "n must be a positive multiple of 128, got %d", n);
   if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must be a positive multiple of 128, got %d", k);
+  if (k > 32768) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must be <= 32768, got %d", k);
   if (total_rows < 0) return fail(ESMOE_ERR_INVALID_ARGUMENT, "total_rows must be >= 0");
   if (out_dtype != ESMOE_OUT_BF16 && out_dtype != ESMOE_OUT_FP16)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "out_dtype must be ESMOE_OUT_BF16 or ESMOE_OUT_FP16");

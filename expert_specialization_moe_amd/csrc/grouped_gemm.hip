@@ -2,19 +2,21 @@
 //
 // One launch serves every expert.  A one-workgroup schedule kernel turns
 // problem_sizes into a list of workgroup tiles (schedule.h); persistent workgroups
-// then pull tiles from an atomic counter.  A workgroup is 4 wavefronts laid out
-// along N; a tile is (MT*16) token rows x (NT*64) weight rows and each wavefront
-// owns NT*16 weight rows of it.
+// of 8 wavefronts then pull tiles from an atomic counter.  A tile is (MT*16) token
+// rows x 256 weight rows.
 //
-// Data movement.  Per 128-wide K block the workgroup loads the token rows and the
-// weight rows of its tile with lane-contiguous 16-byte loads (8 lanes cover one
-// 128-byte row segment, so the texture-address unit sees whole cache lines), keeps
-// them in registers for S-1 K blocks (the global prefetch distance) and then writes
-// them to a double-buffered LDS tile with 144-byte row pitch.  MFMA operand
-// fragments are read back from LDS (16 bytes per lane, conflict-free down a column
-// of rows).  Loading fragments straight from global memory is ~4x slower per CU:
-// a fragment puts consecutive lanes on different rows, i.e. 64 separate 16-byte
-// requests per instruction.
+// Data movement.  Per 128-wide K block the workgroup copies the token rows, the
+// weight rows and the block's scales of its tile from global memory straight into
+// an LDS ring with global_load_lds (no staging registers, no LDS store
+// instructions).  One wavefront instruction moves 8 rows x 128 bytes: 8 consecutive
+// lanes read one row's 128 contiguous bytes, and LDS receives the 64 lanes' 16-byte
+// chunks back to back.  The ring holds 2..4 K blocks depending on the tile height,
+// so up to 3 K blocks of loads are in flight per workgroup.  LDS rows are 128 bytes
+// apart; chunk c of row r is stored in 16-byte slot c ^ ((r >> 1) & 7), which makes
+// the MFMA fragment reads (16 rows x 16 bytes per quarter-wave) bank-conflict free.
+// Loading fragments straight from global memory is ~4x slower per CU: a fragment
+// puts consecutive lanes on different rows, i.e. 64 separate 16-byte requests per
+// instruction.
 //
 // MFMA mapping (v_mfma[_scale]_f32_16x16x128_f8f6f4, both operands e4m3):
 //   * the weight rows ride on the instruction's "A" side and the token rows on its
@@ -42,8 +44,12 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 256;
-constexpr int kLdsRow = 144;  // 128 data bytes + 16 pad: conflict-free 16-byte reads down a column of rows
+constexpr int kThreads = 512;  // 8 wavefronts: two per SIMD, 256 registers each
+constexpr int kWaves = kThreads / 64;
+constexpr int kBN = 256;       // every tile is 256 weight rows wide
+constexpr int kRingBytes = 152 * 1024;  // LDS ring of K-block stages
+constexpr int kMaxKB = 256;             // K <= 32768: per-tile table of weight block scales
+constexpr int kLdsBytes = kRingBytes + 2 * kMaxKB * 4;
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   v8i r;
@@ -52,241 +58,233 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   return r;
 }
 
-// LDS layout of one K-block buffer of a tile: token rows, weight rows, then the block's scales.
-template <int MT, int NT, bool MX>
+// 16-byte slot of chunk c in LDS row r (rows are 128 bytes apart).
+__device__ __forceinline__ int swz(int r, int c) { return c ^ ((r >> 1) & 7); }
+
+// Asynchronous global -> LDS copies: lane i's 16 (4) bytes land at lds_addr + 16*i (4*i).
+// `base` and `lds_addr` are wave-uniform, `voff` is the lane's byte offset from `base`.
+__device__ __forceinline__ void dma16(const void* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void dma4(const void* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void block_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// Shape of a tile with MT*16 token rows and the layout of one ring stage (token rows, weight rows,
+// scales).  Tall tiles (MT >= 8) split the wavefronts 2 (token rows) x 4 (weight rows); short tiles
+// give each of the 8 wavefronts all token rows and 32 weight rows.
+template <int MT, bool MX>
 struct TileGeom {
   static constexpr int BM = MT * 16;
-  static constexpr int BN = NT * 64;
-  static constexpr int kAChunks = BM * 8;   // 16-byte chunks of the token rows of one K block
-  static constexpr int kWChunks = BN * 8;
-  static constexpr int kAPass = (kAChunks + kThreads - 1) / kThreads;
-  static constexpr int kWPass = kWChunks / kThreads;
-  static constexpr int kABytes = BM * kLdsRow;
-  static constexpr int kWBytes = BN * kLdsRow;
-  // scales: fp8-blockwise -> BM floats (sa of the block); mxfp8 -> verbatim 512-byte swizzled tiles,
-  // weight rows first (BN/128 tiles), then token rows (ceil(BM/128) tiles)
-  static constexpr int kSfwChunks = MX ? BN / 4 : 0;
-  static constexpr int kSfaChunks = MX ? ((BM + 127) / 128) * 32 : 0;
-  // every thread stages one scale item (threads past the tile's needs duplicate a valid one), so the
-  // region is sized for 256 items and the pipeline stays free of divergent branches
-  static constexpr int kScaleBytes = MX ? kThreads * 16 : kThreads * 4;
-  static constexpr int kBufBytes = kABytes + kWBytes + ((kScaleBytes + 15) & ~15);
-  static_assert(kWChunks % kThreads == 0, "weight tile must fill whole passes");
-  static_assert(kSfwChunks + kSfaChunks <= kThreads, "one scale chunk per thread");
+  static constexpr int kWavesM = MT >= 8 ? 2 : 1;
+  static constexpr int kWavesN = kWaves / kWavesM;
+  static constexpr int MTW = MT / kWavesM;          // row tiles per wavefront
+  static constexpr int NTW = kBN / 16 / kWavesN;    // weight-row tiles per wavefront
+  static constexpr int kABytes = BM * 128;
+  static constexpr int kWBytes = kBN * 128;
+  // scales of one K block: fp8-blockwise -> 256 floats (sa of the tile's rows); mxfp8 -> verbatim
+  // 512-byte swizzled scale tiles, 2 for the weight rows then up to 2 for the token rows
+  static constexpr int kScaleBytes = MX ? 2048 : 1024;
+  static constexpr int kStageBytes = kABytes + kWBytes + kScaleBytes;
+  static constexpr int kNBuf = kRingBytes / kStageBytes >= 4 ? 4 : kRingBytes / kStageBytes;
+  static constexpr int kABlocks = BM / 8;                               // 8-row copy blocks of the token tile
+  static constexpr int kACopies = kABlocks >= kWaves ? kABlocks / kWaves : 1;  // per wavefront
+  static constexpr int kWCopies = kBN / 8 / kWaves;                     // 4
+  static constexpr int kCopiesPerStage = kACopies + kWCopies + 1;       // + 1 scale copy
+  static_assert(kNBuf >= 2, "ring too small");
 };
 
-// Largest LDS footprint over the compiled shapes (two buffers).
-constexpr int kLdsBytes = 2 * ((128 + 256) * kLdsRow + 4096);
-
-// One K block of a tile in flight between global memory and LDS.
-template <int MT, int NT, bool MX>
-struct TileStage {
-  using G = TileGeom<MT, NT, MX>;
-  v4i a[G::kAPass];
-  v4i w[G::kWPass];
-  float sa;   // fp8-blockwise: sa[row of this thread][kb] (threads < BM)
-  float sb;   // fp8-blockwise: sb[e][n-block of this wavefront][kb]
-  v4i sf;     // mxfp8: this thread's 16-byte chunk of the swizzled scale tiles
-};
-
-template <int MT, int NT, bool MX, int S>
+template <int MT, bool MX>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds) {
-  using G = TileGeom<MT, NT, MX>;
-  static_assert(2 * G::kBufBytes <= kLdsBytes, "LDS budget");
+  using G = TileGeom<MT, MX>;
+  constexpr int MTW = G::MTW, NTW = G::NTW, NBUF = G::kNBuf;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / G::kWavesN, wn = wave % G::kWavesN;
   const int r = lane & 15;
   const int gq = lane >> 4;
   const int K = g.k, N = g.n, KB = K >> 7;
   const long row_base = g.expert_offsets[e];
-  const int nw0 = n0 + wave * (NT * 16);
-  const bool wave_active = nw0 < N;
+  const int nw = wn * (NTW * 16);          // first weight row of this wavefront inside the tile
+  const int mw = wm * (MTW * 16);          // first token row of this wavefront inside the tile
+  const bool wave_active = n0 + nw < N;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+  float* s_sb = (float*)(lds + kRingBytes);  // [2][kMaxKB] weight block scales of the tile's two 128-column blocks
 
-  // staging map: chunk c -> row c/8, 16-byte column c%8 (8 consecutive lanes = one 128-byte row
-  // segment).  Addresses are a wave-uniform 64-bit base plus one 32-bit offset per pass.
-  const int srow = tid >> 3, scol = tid & 7;       // pass p handles tile row srow + 32*p
+  // ---- copy plan: this lane's global byte offsets (from wave-uniform bases) -----------------
+  const int crow = lane >> 3, cslot = lane & 7;    // lane -> (row in 8-row block, 16-byte slot)
   const uint8_t* a_base = (const uint8_t*)g.a + (row_base + m0) * K;
   const uint8_t* w_base = (const uint8_t*)g.b + ((long)e * N + n0) * K;
-  // (a token tile shorter than 32 rows is staged twice by the two halves of the workgroup: same
-  // bytes to the same place, which keeps every thread on the same instruction stream)
-  const int arow0 = srow & (G::BM < 32 ? G::BM - 1 : 31);
-  uint32_t aoff[G::kAPass];
+  uint32_t aoff[G::kACopies];
+  uint32_t alds[G::kACopies];
 #pragma unroll
-  for (int p = 0; p < G::kAPass; p++) {
-    int row = arow0 + 32 * p;
-    if (row > M - 1 - m0) row = M - 1 - m0;
-    aoff[p] = (uint32_t)row * (uint32_t)K + scol * 16;
+  for (int i = 0; i < G::kACopies; i++) {
+    const int blk = (wave + kWaves * i) % G::kABlocks;   // short tiles are copied by several wavefronts
+    const int row = blk * 8 + crow;
+    int grow = row;
+    if (grow > M - 1 - m0) grow = M - 1 - m0;
+    aoff[i] = (uint32_t)grow * (uint32_t)K + swz(row, cslot) * 16;
+    alds[i] = blk * 1024;
   }
-  uint32_t woff[G::kWPass];
+  uint32_t woff[G::kWCopies];
 #pragma unroll
-  for (int p = 0; p < G::kWPass; p++) {
-    int row = srow + 32 * p;
-    if (row > N - 1 - n0) row = N - 1 - n0;
-    woff[p] = (uint32_t)row * (uint32_t)K + scol * 16;
+  for (int i = 0; i < G::kWCopies; i++) {
+    const int row = (wave * G::kWCopies + i) * 8 + crow;
+    int grow = row;
+    if (grow > N - 1 - n0) grow = N - 1 - n0;
+    woff[i] = (uint32_t)grow * (uint32_t)K + swz(row, cslot) * 16;
   }
-  const int sdst = srow * kLdsRow + scol * 16;     // LDS offset of pass 0; pass p adds 32 rows
-  const int adst = arow0 * kLdsRow + scol * 16;
-  constexpr int kScaleOff = G::kABytes + G::kWBytes;
-  const float* sa_src = nullptr;
-  const float* sb_src = nullptr;
-  const uint8_t* sf_src = nullptr;
+  const uint32_t wlds = G::kABytes + wave * G::kWCopies * 1024;
+  // scales
+  const uint8_t* sc_base;
+  uint32_t scoff, sclds;
   if constexpr (!MX) {
-    int grow = m0 + tid;
-    if (grow > M - 1) grow = M - 1;
-    sa_src = g.sa + (row_base + grow) * KB;
-    sb_src = g.sb + ((long)e * (N >> 7) + ((wave_active ? nw0 : 0) >> 7)) * KB;
+    int row = (wave & 3) * 64 + lane;                   // wavefronts 4..7 repeat rows 0..255
+    if (row > M - 1 - m0) row = M - 1 - m0;
+    sc_base = (const uint8_t*)(g.sa + (row_base + m0) * KB);
+    scoff = (uint32_t)row * (uint32_t)KB * 4;
+    sclds = G::kABytes + G::kWBytes + (wave & 3) * 256;
   } else {
     const int kc = K >> 5;
-    if (tid < G::kSfwChunks) {
-      int blk = (n0 >> 7) + (tid >> 5);
+    int blk;
+    if ((wave & 1) == 0) {  // even wavefronts: the two weight scale tiles
+      blk = (n0 >> 7) + (lane >> 5);
       if (blk * 128 >= N) blk = n0 >> 7;
-      sf_src = g.sfb + (long)e * N * kc + (long)blk * KB * 512 + (tid & 31) * 16;
-    } else {
-      int j = tid - G::kSfwChunks;
-      int blk = (m0 >> 7) + (j >> 5);
-      if (j >= G::kSfaChunks || blk * 128 >= M) blk = m0 >> 7;
-      sf_src = g.sfa + (long)g.blockscale_offsets[e] * kc + (long)blk * KB * 512 + (j & 31) * 16;
+      sc_base = g.sfb + (long)e * N * kc;
+    } else {                // odd wavefronts: the token scale tile(s)
+      blk = (m0 >> 7) + (lane >> 5);
+      if (blk * 128 >= M) blk = m0 >> 7;
+      sc_base = g.sfa + (long)g.blockscale_offsets[e] * kc;
     }
+    scoff = (uint32_t)blk * (uint32_t)KB * 512 + (lane & 31) * 16;
+    sclds = G::kABytes + G::kWBytes + (wave & 1) * 1024;
   }
 
-  const int frag_off = r * kLdsRow + gq * 16;
-  const int wfrag_off = G::kABytes + wave * (NT * 16) * kLdsRow + frag_off;
-
-  v4f acc[NT][MT];
-#pragma unroll
-  for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++) acc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
-
-  TileStage<MT, NT, MX> st[S];
-
-  auto load = [&](TileStage<MT, NT, MX>& t, int kb) {
+  auto issue = [&](int kb, int buf) {
+    const uint32_t sb = lds0 + buf * G::kStageBytes;
     const uint8_t* ab = a_base + (long)kb * 128;
     const uint8_t* wb = w_base + (long)kb * 128;
 #pragma unroll
-    for (int p = 0; p < G::kAPass; p++) {
-      t.a[p] = *(const v4i*)(ab + aoff[p]);
-    }
+    for (int i = 0; i < G::kACopies; i++) dma16(ab, aoff[i], sb + alds[i]);
 #pragma unroll
-    for (int p = 0; p < G::kWPass; p++) t.w[p] = *(const v4i*)(wb + woff[p]);
+    for (int i = 0; i < G::kWCopies; i++) dma16(wb, woff[i], sb + wlds + i * 1024);
     if constexpr (!MX) {
-      t.sa = sa_src[kb];
-      t.sb = sb_src[kb];
+      dma4(sc_base + (long)kb * 4, scoff, sb + sclds);
     } else {
-      t.sf = *(const v4i*)(sf_src + (long)kb * 512);
+      dma16(sc_base + (long)kb * 512, scoff, sb + sclds);
     }
   };
-  auto store = [&](const TileStage<MT, NT, MX>& t, int buf) {
-    uint8_t* lb = lds + buf * G::kBufBytes;
+
+  // ---- fragment read plan ----------------------------------------------------------------
+  // token fragment of row tile mt: LDS row ra = mw + mt*16 + r, chunks gq and gq+4
+  // (mw, mt*16 are multiples of 16, so the slot permutation depends on r only)
+  const int slot_lo = swz(r, gq), slot_hi = swz(r, gq + 4);
+  const int afrag_lo = (mw + r) * 128 + slot_lo * 16, afrag_hi = (mw + r) * 128 + slot_hi * 16;
+  const int wfrag_lo = G::kABytes + (nw + r) * 128 + slot_lo * 16, wfrag_hi = G::kABytes + (nw + r) * 128 + slot_hi * 16;
+  constexpr int kScaleOff = G::kABytes + G::kWBytes;
+  const float* sb_tab = s_sb + (nw >> 7) * kMaxKB;
+
+  v4f acc[NTW][MTW];
 #pragma unroll
-    for (int p = 0; p < G::kAPass; p++) *(v4i*)(lb + adst + p * 32 * kLdsRow) = t.a[p];
+  for (int nt = 0; nt < NTW; nt++)
 #pragma unroll
-    for (int p = 0; p < G::kWPass; p++) *(v4i*)(lb + sdst + G::kABytes + p * 32 * kLdsRow) = t.w[p];
-    if constexpr (!MX) {
-      *(float*)(lb + kScaleOff + tid * 4) = t.sa;
-    } else {
-      *(v4i*)(lb + kScaleOff + tid * 16) = t.sf;
+    for (int mt = 0; mt < MTW; mt++) acc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  auto compute = [&](int kb, int buf) {
+    const uint8_t* lb = lds + buf * G::kStageBytes;
+    v8i wf[NTW];
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      wf[nt] = join(*(const v4i*)(lb + wfrag_lo + nt * 2048), *(const v4i*)(lb + wfrag_hi + nt * 2048));
     }
-  };
-  auto compute = [&](const TileStage<MT, NT, MX>& t, int buf) {
-    const uint8_t* lb = lds + buf * G::kBufBytes;
-    v8i wf[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      wf[nt] = join(*(const v4i*)(lb + wfrag_off + nt * 16 * kLdsRow), *(const v4i*)(lb + wfrag_off + nt * 16 * kLdsRow + 64));
-    }
-    int sfw[MX ? NT : 1];
+    int sfw[MX ? NTW : 1];
+    float sbv = 0.f;
     if constexpr (MX) {
 #pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        int nl = wave * (NT * 16) + nt * 16 + r;  // weight row inside the tile
+      for (int nt = 0; nt < NTW; nt++) {
+        int nl = nw + nt * 16 + r;  // weight row inside the tile
         uint32_t d = *(const uint32_t*)(lb + kScaleOff + (nl >> 7) * 512 + (nl & 31) * 16 + ((nl & 127) >> 5) * 4);
         sfw[nt] = (int)(d >> (gq * 8));
       }
+    } else {
+      sbv = sb_tab[kb];
     }
-    v4i af[2][2];
-    af[0][0] = *(const v4i*)(lb + frag_off);
-    af[0][1] = *(const v4i*)(lb + frag_off + 64);
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-      if (mt + 1 < MT) {
-        af[(mt + 1) & 1][0] = *(const v4i*)(lb + frag_off + (mt + 1) * 16 * kLdsRow);
-        af[(mt + 1) & 1][1] = *(const v4i*)(lb + frag_off + (mt + 1) * 16 * kLdsRow + 64);
-      }
-      v8i afr = join(af[mt & 1][0], af[mt & 1][1]);
+    for (int mt = 0; mt < MTW; mt++) {
+      v8i afr = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + afrag_hi + mt * 2048));
       if constexpr (!MX) {
-        float sc = *(const float*)(lb + kScaleOff + (mt * 16 + r) * 4) * t.sb;
-        v4f tmp[NT];
+        float sc = *(const float*)(lb + kScaleOff + (mw + mt * 16 + r) * 4) * sbv;
+        v4f tmp[NTW];
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
+        for (int nt = 0; nt < NTW; nt++) {
           tmp[nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], afr, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
         }
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
+        for (int nt = 0; nt < NTW; nt++) {
 #pragma unroll
           for (int i = 0; i < 4; i++) acc[nt][mt][i] = __builtin_fmaf(tmp[nt][i], sc, acc[nt][mt][i]);
         }
       } else {
-        int ml = (m0 & 127) + mt * 16 + r;  // token row inside its 128-row scale tile(s)
-        uint32_t d = *(const uint32_t*)(lb + kScaleOff + G::kSfwChunks * 16 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4);
+        int ml = (m0 & 127) + mw + mt * 16 + r;  // token row inside its 128-row scale tile(s)
+        uint32_t d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4);
         int sfa = (int)(d >> (gq * 8));
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
+        for (int nt = 0; nt < NTW; nt++) {
           acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], afr, acc[nt][mt], 0, 0, 0, sfw[nt], 0, sfa);
         }
       }
     }
   };
 
-  // prologue: S-1 K blocks in flight, the first one into LDS buffer 0
+  // ---- pipeline --------------------------------------------------------------------------
+  // prologue: NBUF-1 K blocks in flight
 #pragma unroll
-  for (int j = 0; j < S - 1; j++) {
-    if (j < KB) load(st[j], j);
+  for (int s = 0; s < NBUF - 1; s++) {
+    if (s < KB) issue(s, s);
   }
-  store(st[0], 0);
-  __syncthreads();
+  if constexpr (!MX) {
+    // weight block scales of the whole tile (2 column blocks x KB), read back after the first barrier
+    const int blk = tid >> 8, kbi = tid & 255;
+    int nb = (n0 >> 7) + blk;
+    if (nb * 128 >= N) nb = n0 >> 7;
+    if (kbi < KB) s_sb[blk * kMaxKB + kbi] = g.sb[((long)e * (N >> 7) + nb) * KB + kbi];
+  }
+  if (KB >= NBUF - 1) wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>(); else wait_vmcnt<0>();
+  block_barrier();
 
-  // steady state: branch-free so that the outstanding-load counts stay exact
-  int kb0 = 0;
-  for (; kb0 + 2 * S - 2 < KB; kb0 += S) {
-#pragma unroll
-    for (int j = 0; j < S; j++) {
-      const int kb = kb0 + j;
-      load(st[(j + S - 1) % S], kb + S - 1);
-      __builtin_amdgcn_sched_barrier(0);  // keep the phases in program order: the scheduler would
-      compute(st[j], kb & 1);             // otherwise overlap all stages' live ranges and spill
-      __builtin_amdgcn_sched_barrier(0);
-      store(st[(j + 1) % S], (kb + 1) & 1);
-      __syncthreads();
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-  // drain: at most 2S-2 K blocks left
-#pragma unroll
-  for (int t = 0; t < 2; t++) {
-#pragma unroll
-    for (int j = 0; j < S; j++) {
-      const int kb = kb0 + t * S + j;
-      if (kb < KB) {
-        if (kb + S - 1 < KB) load(st[(j + S - 1) % S], kb + S - 1);
-        compute(st[j], kb & 1);
-        if (kb + 1 < KB) store(st[(j + 1) % S], (kb + 1) & 1);
-        __syncthreads();
-      }
-    }
+  int buf = 0, nbuf = NBUF - 1;  // ring slots of K block kb and of K block kb + NBUF - 1
+  for (int kb = 0; kb < KB; kb++) {
+    const bool more = kb + NBUF - 1 < KB;
+    if (more) issue(kb + NBUF - 1, nbuf);
+    compute(kb, buf);
+    // K block kb+1 must have landed (all but the newest NBUF-2 stages), and every wavefront must be
+    // done reading slot `buf` before the next iteration's copies overwrite it
+    if (more) wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>(); else wait_vmcnt<0>();
+    block_barrier();
+    buf = buf + 1 == NBUF ? 0 : buf + 1;
+    nbuf = nbuf + 1 == NBUF ? 0 : nbuf + 1;
   }
 
-  // epilogue: lane holds columns nw0 + nt*16 + 4*gq + [0,4) of token row m0 + mt*16 + r
+  // epilogue: lane holds columns n0 + nw + nt*16 + 4*gq + [0,4) of token row m0 + mw + mt*16 + r
   if (wave_active) {
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-      int m = m0 + mt * 16 + r;
+    for (int mt = 0; mt < MTW; mt++) {
+      int m = m0 + mw + mt * 16 + r;
       if (m < M) {
         long orow = (row_base + m) * (long)N;
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-          int n = nw0 + nt * 16 + gq * 4;
+        for (int nt = 0; nt < NTW; nt++) {
+          int n = n0 + nw + nt * 16 + gq * 4;
           if (g.out_dtype == 0) {
             *(bf16x4*)((__bf16*)g.out + orow + n) = __builtin_convertvector(acc[nt][mt], bf16x4);
           } else {
@@ -338,20 +336,13 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
   }
 }
 
-// (MT, NT) tile shapes compiled into the persistent kernel.
+// Tile heights (MT * 16 rows) compiled into the persistent kernel.
 #ifndef ESMOE_VARIANTS
-#define ESMOE_VARIANTS \
-  ESMOE_CASE(1, 4) ESMOE_CASE(2, 4) ESMOE_CASE(4, 4) ESMOE_CASE(8, 4) ESMOE_CASE(16, 2)
-#endif
-#ifndef ESMOE_STAGES
-#define ESMOE_STAGES 3
-#endif
-#ifndef ESMOE_WAVES_PER_SIMD
-#define ESMOE_WAVES_PER_SIMD 1
+#define ESMOE_VARIANTS ESMOE_CASE(1) ESMOE_CASE(2) ESMOE_CASE(4) ESMOE_CASE(8)
 #endif
 
 template <bool MX>
-__global__ void __launch_bounds__(kThreads, ESMOE_WAVES_PER_SIMD) grouped_gemm_kernel(GemmArgs g) {
+__global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
   __shared__ int s_item;
   int* ws = g.ws;
@@ -373,9 +364,9 @@ __global__ void __launch_bounds__(kThreads, ESMOE_WAVES_PER_SIMD) grouped_gemm_k
     const int e = order[lo];
     const int M = g.problem_sizes[e * 3];
     const TileCoord t = sched_decode(item - item_start[lo], M, g.n, g.policy);
-    const int key = t.mt * 8 + t.nt;
-#define ESMOE_CASE(MT_, NT_) \
-  case (MT_) * 8 + (NT_): gemm_tile<MT_, NT_, MX, ((MT_) >= 16 ? 2 : ESMOE_STAGES)>(g, e, M, t.m0, t.n0, lds); break;
+    const int key = t.mt;
+#define ESMOE_CASE(MT_) \
+  case (MT_): gemm_tile<MT_, MX>(g, e, M, t.m0, t.n0, lds); break;
     switch (key) {
       ESMOE_VARIANTS
       default: break;

@@ -42,8 +42,8 @@ ESMOE_HD int sched_cover_mt(int rows, int max_mt) {
   return mt;
 }
 
-// Compiled shapes: MT in {1, 2, 4, 8} are 256 columns wide (NT = 4), MT = 16 is 128 wide (NT = 2).
-ESMOE_HD int sched_nt_for(int mt, const SchedPolicy&) { return mt >= 16 ? 2 : 4; }
+// Every compiled shape is 256 columns wide (NT = 4 units of 64).
+ESMOE_HD int sched_nt_for(int, const SchedPolicy&) { return 4; }
 
 ESMOE_HD int sched_ntiles(int n, int nt) { return (n + nt * 64 - 1) / (nt * 64); }
 
