@@ -64,10 +64,13 @@ int env_int(const char* name, int dflt) {
 }
 
 // Default schedule policy; ESMOE_* environment variables override single fields (tuning aid).
-esmoe::SchedPolicy make_policy(int force_bm) {
+esmoe::SchedPolicy make_policy(int force_bm, int mx) {
   esmoe::SchedPolicy p;
   p.force_mt = force_bm / 16;
-  p.big_mt = env_int("ESMOE_BIG_MT", 8);
+  // 256-row tiles need 128 accumulator registers per lane, which the mxfp8 kernel can afford (it
+  // accumulates inside the MFMA); the fp8-blockwise kernel also needs VALU temporaries for its
+  // scale-and-accumulate step and is fastest with 128-row tiles
+  p.big_mt = env_int("ESMOE_BIG_MT", mx ? 16 : 8);
   p.order = env_int("ESMOE_ORDER", 0);
   return p;
 }
@@ -83,8 +86,9 @@ int check_common(const void* out, const void* a, const void* b, const int32_t* p
   if (total_rows < 0) return fail(ESMOE_ERR_INVALID_ARGUMENT, "total_rows must be >= 0");
   if (out_dtype != ESMOE_OUT_BF16 && out_dtype != ESMOE_OUT_FP16)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "out_dtype must be ESMOE_OUT_BF16 or ESMOE_OUT_FP16");
-  if (force_bm != 0 && force_bm != 16 && force_bm != 32 && force_bm != 64 && force_bm != 128 && force_bm != 256)
-    return fail(ESMOE_ERR_INVALID_ARGUMENT, "force_bm must be 0, 16, 32, 64, 128 or 256, got %d", force_bm);
+  if (force_bm != 0 && force_bm != 16 && force_bm != 32 && force_bm != 64 && force_bm != 128 && force_bm != 192 &&
+      force_bm != 256)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "force_bm must be 0, 16, 32, 64, 128, 192 or 256, got %d", force_bm);
   if (!workspace || workspace_bytes < esmoe_gemm_workspace_bytes(num_experts))
     return fail(ESMOE_ERR_WORKSPACE_TOO_SMALL, "workspace of %zu bytes is smaller than the %zu required",
                 workspace_bytes, esmoe_gemm_workspace_bytes(num_experts));
@@ -99,7 +103,7 @@ int launch_gemm(esmoe::GemmArgs& g, int mx, int force_bm, void* stream) {
   DeviceInfo info;
   int rc = current_device_info(&info);
   if (rc) return rc;
-  g.policy = make_policy(force_bm);
+  g.policy = make_policy(force_bm, mx);
   int grid = info.cus * env_int("ESMOE_WGS_PER_CU", 1);
   rc = esmoe_launch_grouped_gemm(&g, mx, grid, (hipStream_t)stream);
   if (rc) return fail(rc, "grouped GEMM launch failed: %s", hipGetErrorString((hipError_t)rc));
@@ -183,7 +187,7 @@ int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int 
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS || n <= 0 || n % 128)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_schedule");
-  const esmoe::SchedPolicy p = make_policy(force_bm);
+  const esmoe::SchedPolicy p = make_policy(force_bm, 0);
   int32_t* item_start = ws_host + esmoe::ws_item_start(num_experts);
   int32_t* order = ws_host + esmoe::ws_order(num_experts);
   // same ranking as the device schedule kernel: most rows first, ties by expert index
@@ -215,7 +219,7 @@ int esmoe_host_decode_item(const int32_t* problem_sizes_host, const int32_t* ws_
                            int force_bm, int item, int32_t* out5) {
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || !out5) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null pointer");
-  const esmoe::SchedPolicy p = make_policy(force_bm);
+  const esmoe::SchedPolicy p = make_policy(force_bm, 0);
   const int32_t* item_start = ws_host + esmoe::ws_item_start(num_experts);
   const int32_t* order = ws_host + esmoe::ws_order(num_experts);
   if (item < 0 || item >= ws_host[esmoe::kWsTotal]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "item out of range");

@@ -47,9 +47,10 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 512;  // 8 wavefronts: two per SIMD, 256 registers each
 constexpr int kWaves = kThreads / 64;
 constexpr int kBN = 256;       // every tile is 256 weight rows wide
-constexpr int kRingBytes = 152 * 1024;  // LDS ring of K-block stages
+constexpr int kRingBytes = 148 * 1024;  // LDS ring of K-block stages
 constexpr int kMaxKB = 256;             // K <= 32768: per-tile table of weight block scales
-constexpr int kLdsBytes = kRingBytes + 2 * kMaxKB * 4;
+constexpr int kSaChunkBytes = 2 * 256 * 16;  // fp8-blockwise: two buffers of [256 rows][4 K blocks] activation scales
+constexpr int kLdsBytes = kRingBytes + 2 * kMaxKB * 4 + kSaChunkBytes;
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   v8i r;
@@ -120,40 +121,33 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   const bool wave_active = n0 + nw < N;
   const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
   float* s_sb = (float*)(lds + kRingBytes);  // [2][kMaxKB] weight block scales of the tile's two 128-column blocks
+  constexpr int kSaChunkOff = kRingBytes + 2 * kMaxKB * 4;
 
-  // ---- copy plan: this lane's global byte offsets (from wave-uniform bases) -----------------
-  const int crow = lane >> 3, cslot = lane & 7;    // lane -> (row in 8-row block, 16-byte slot)
+  // ---- copy plan -------------------------------------------------------------------------
+  // A copy instruction moves the 8-row block `blk` of the stage: lane -> (row crow, slot cslot), and
+  // the slot holds chunk cslot ^ ((row >> 1) & 7) = cslot ^ (crow >> 1) ^ 4*(blk & 1).  So two
+  // per-lane offsets (even / odd block) serve every interior block of both operands; the block's
+  // first row goes into the wave-uniform base.  Blocks that cross the end of the expert's rows
+  // take a slower path that clamps the row per lane.
+  const int crow = lane >> 3, cslot = lane & 7;
+  const uint32_t ro_even = (uint32_t)crow * (uint32_t)K + ((cslot ^ (crow >> 1)) << 4);
+  const uint32_t ro_odd = ro_even ^ 64u;
   const uint8_t* a_base = (const uint8_t*)g.a + (row_base + m0) * K;
   const uint8_t* w_base = (const uint8_t*)g.b + ((long)e * N + n0) * K;
-  uint32_t aoff[G::kACopies];
-  uint32_t alds[G::kACopies];
-#pragma unroll
-  for (int i = 0; i < G::kACopies; i++) {
-    const int blk = (wave + kWaves * i) % G::kABlocks;   // short tiles are copied by several wavefronts
-    const int row = blk * 8 + crow;
-    int grow = row;
-    if (grow > M - 1 - m0) grow = M - 1 - m0;
-    aoff[i] = (uint32_t)grow * (uint32_t)K + swz(row, cslot) * 16;
-    alds[i] = blk * 1024;
-  }
-  uint32_t woff[G::kWCopies];
-#pragma unroll
-  for (int i = 0; i < G::kWCopies; i++) {
-    const int row = (wave * G::kWCopies + i) * 8 + crow;
-    int grow = row;
-    if (grow > N - 1 - n0) grow = N - 1 - n0;
-    woff[i] = (uint32_t)grow * (uint32_t)K + swz(row, cslot) * 16;
-  }
-  const uint32_t wlds = G::kABytes + wave * G::kWCopies * 1024;
+  const int a_last = M - 1 - m0;   // last valid token row of the tile
   // scales
   const uint8_t* sc_base;
   uint32_t scoff, sclds;
+  // fp8-blockwise activation scales sa[row][kb]: when KB is a multiple of 4 they are fetched 4 K blocks
+  // at a time (16 bytes per row, one copy per wavefront every 4th K block, double-buffered outside
+  // the ring); otherwise one float per row and K block travels with every stage.
+  const bool sa4 = !MX && (KB & 3) == 0;
   if constexpr (!MX) {
     int row = (wave & 3) * 64 + lane;                   // wavefronts 4..7 repeat rows 0..255
-    if (row > M - 1 - m0) row = M - 1 - m0;
+    if (row > a_last) row = a_last;
     sc_base = (const uint8_t*)(g.sa + (row_base + m0) * KB);
     scoff = (uint32_t)row * (uint32_t)KB * 4;
-    sclds = G::kABytes + G::kWBytes + (wave & 3) * 256;
+    sclds = sa4 ? kSaChunkOff + (wave & 3) * 1024 : G::kABytes + G::kWBytes + (wave & 3) * 256;
   } else {
     const int kc = K >> 5;
     int blk;
@@ -170,16 +164,31 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     sclds = G::kABytes + G::kWBytes + (wave & 1) * 1024;
   }
 
+  // scales of K blocks 4c .. 4c+3 into chunk buffer c & 1
+  auto issue_sa_chunk = [&](int c) { dma16(sc_base + (long)c * 16, scoff, lds0 + sclds + (c & 1) * 4096); };
   auto issue = [&](int kb, int buf) {
     const uint32_t sb = lds0 + buf * G::kStageBytes;
     const uint8_t* ab = a_base + (long)kb * 128;
     const uint8_t* wb = w_base + (long)kb * 128;
 #pragma unroll
-    for (int i = 0; i < G::kACopies; i++) dma16(ab, aoff[i], sb + alds[i]);
+    for (int i = 0; i < G::kACopies; i++) {
+      const int blk = (wave + kWaves * i) % G::kABlocks;   // short tiles are copied by several wavefronts
+      if (blk * 8 + 7 <= a_last) {
+        dma16(ab + (long)blk * 8 * K, (blk & 1) ? ro_odd : ro_even, sb + blk * 1024);
+      } else {
+        int row = blk * 8 + crow;
+        int grow = row > a_last ? a_last : row;
+        dma16(ab, (uint32_t)grow * (uint32_t)K + (swz(row, cslot) << 4), sb + blk * 1024);
+      }
+    }
 #pragma unroll
-    for (int i = 0; i < G::kWCopies; i++) dma16(wb, woff[i], sb + wlds + i * 1024);
+    for (int i = 0; i < G::kWCopies; i++) {
+      const int blk = wave * G::kWCopies + i;
+      const int src = n0 + blk * 8 < N ? blk : i;          // past the last weight row: copy valid rows instead
+      dma16(wb + (long)src * 8 * K, (blk & 1) ? ro_odd : ro_even, sb + G::kABytes + blk * 1024);
+    }
     if constexpr (!MX) {
-      dma4(sc_base + (long)kb * 4, scoff, sb + sclds);
+      if (!sa4) dma4(sc_base + (long)kb * 4, scoff, sb + sclds);
     } else {
       dma16(sc_base + (long)kb * 512, scoff, sb + sclds);
     }
@@ -188,11 +197,16 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // ---- fragment read plan ----------------------------------------------------------------
   // token fragment of row tile mt: LDS row ra = mw + mt*16 + r, chunks gq and gq+4
   // (mw, mt*16 are multiples of 16, so the slot permutation depends on r only)
-  const int slot_lo = swz(r, gq), slot_hi = swz(r, gq + 4);
-  const int afrag_lo = (mw + r) * 128 + slot_lo * 16, afrag_hi = (mw + r) * 128 + slot_hi * 16;
-  const int wfrag_lo = G::kABytes + (nw + r) * 128 + slot_lo * 16, wfrag_hi = G::kABytes + (nw + r) * 128 + slot_hi * 16;
+  // (the high chunk gq+4 sits 4 slots = 64 bytes away in the xor order)
+  const int afrag_lo = (mw + r) * 128 + swz(r, gq) * 16;
+  const int wfrag_lo = G::kABytes + (nw + r) * 128 + swz(r, gq) * 16;
   constexpr int kScaleOff = G::kABytes + G::kWBytes;
   const float* sb_tab = s_sb + (nw >> 7) * kMaxKB;
+  // mxfp8: per-lane bases of the scale dwords (weight rows nw + r, token rows mw + r of a tall tile)
+  const int sfw_lane = kScaleOff + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16;
+  const int sfa_lane = kScaleOff + 1024 + (mw >> 7) * 512 + ((mw & 127) >> 5) * 4 + r * 16;
+  const int sa_lane = kScaleOff + (mw + r) * 4;   // fp8-blockwise: float sa of token row mw + r
+  const int sa4_lane = kSaChunkOff + (mw + r) * 16;
 
   v4f acc[NTW][MTW];
 #pragma unroll
@@ -205,15 +219,17 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     v8i wf[NTW];
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
-      wf[nt] = join(*(const v4i*)(lb + wfrag_lo + nt * 2048), *(const v4i*)(lb + wfrag_hi + nt * 2048));
+      wf[nt] = join(*(const v4i*)(lb + wfrag_lo + nt * 2048), *(const v4i*)(lb + (wfrag_lo ^ 64) + nt * 2048));
     }
     int sfw[MX ? NTW : 1];
     float sbv = 0.f;
     if constexpr (MX) {
+      // scale dword of weight row nl = nw + nt*16 + r inside the swizzled 512-byte tiles: nw is a
+      // multiple of NTW*16, so the tile / quarter / row parts of nt are compile-time offsets
 #pragma unroll
       for (int nt = 0; nt < NTW; nt++) {
-        int nl = nw + nt * 16 + r;  // weight row inside the tile
-        uint32_t d = *(const uint32_t*)(lb + kScaleOff + (nl >> 7) * 512 + (nl & 31) * 16 + ((nl & 127) >> 5) * 4);
+        constexpr int kQuarter = NTW == 4 ? 1 : 0;  // NTW = 4: nt/2 selects the 32-row quarter
+        uint32_t d = *(const uint32_t*)(lb + sfw_lane + (nt & 1) * 256 + (kQuarter ? (nt >> 1) * 4 : 0));
         sfw[nt] = (int)(d >> (gq * 8));
       }
     } else {
@@ -221,9 +237,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     }
 #pragma unroll
     for (int mt = 0; mt < MTW; mt++) {
-      v8i afr = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + afrag_hi + mt * 2048));
+      v8i afr = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + (afrag_lo ^ 64) + mt * 2048));
       if constexpr (!MX) {
-        float sc = *(const float*)(lb + kScaleOff + (mw + mt * 16 + r) * 4) * sbv;
+        float sc = (sa4 ? *(const float*)(lds + sa4_lane + ((kb >> 2) & 1) * 4096 + (kb & 3) * 4 + mt * 256)
+                        : *(const float*)(lb + sa_lane + mt * 64)) * sbv;
         v4f tmp[NTW];
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++) {
@@ -235,19 +252,33 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
           for (int i = 0; i < 4; i++) acc[nt][mt][i] = __builtin_fmaf(tmp[nt][i], sc, acc[nt][mt][i]);
         }
       } else {
-        int ml = (m0 & 127) + mw + mt * 16 + r;  // token row inside its 128-row scale tile(s)
-        uint32_t d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4);
+        uint32_t d;
+        if constexpr (MT == 8 || MT == 16) {
+          // tall tiles start on a 128-row boundary and a wavefront's rows start on a multiple of its
+          // own height (64 or 128): row tile mt adds compile-time offsets
+          d = *(const uint32_t*)(lb + sfa_lane + (mt >> 3) * 512 + (mt & 1) * 256 + ((mt & 7) >> 1) * 4);
+        } else if constexpr (MT == 12) {
+          int ml = (m0 & 127) + mw + mt * 16 + r;
+          d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4);
+        } else {
+          int ml = (m0 & 127) + mt * 16 + r;  // token row inside its 128-row scale tile
+          d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml & 31) * 16 + (ml >> 5) * 4);
+        }
         int sfa = (int)(d >> (gq * 8));
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++) {
           acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], afr, acc[nt][mt], 0, 0, 0, sfw[nt], 0, sfa);
         }
       }
+#ifdef ESMOE_MT_SCHED_BARRIER
+      if constexpr (MTW >= 8) __builtin_amdgcn_sched_barrier(0);
+#endif
     }
   };
 
   // ---- pipeline --------------------------------------------------------------------------
   // prologue: NBUF-1 K blocks in flight
+  if (sa4) issue_sa_chunk(0);
 #pragma unroll
   for (int s = 0; s < NBUF - 1; s++) {
     if (s < KB) issue(s, s);
@@ -259,17 +290,32 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     if (nb * 128 >= N) nb = n0 >> 7;
     if (kbi < KB) s_sb[blk * kMaxKB + kbi] = g.sb[((long)e * (N >> 7) + nb) * KB + kbi];
   }
-  if (KB >= NBUF - 1) wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>(); else wait_vmcnt<0>();
+  // copies outstanding per in-flight stage (the chunked scale copies are older than any stage that
+  // may still be in flight when their data is needed, see the loop)
+  if (KB < NBUF - 1) wait_vmcnt<0>();
+  else if (sa4) wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1)>();
+  else wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>();
   block_barrier();
 
   int buf = 0, nbuf = NBUF - 1;  // ring slots of K block kb and of K block kb + NBUF - 1
   for (int kb = 0; kb < KB; kb++) {
     const bool more = kb + NBUF - 1 < KB;
+    // next chunk of activation scales, 4 K blocks before its first use: at least 3 end-of-iteration
+    // waits lie in between and each of them retires everything older than the newest NBUF-2 stages
+    if (sa4 && (kb & 3) == 0 && kb + 4 < KB) issue_sa_chunk((kb >> 2) + 1);
     if (more) issue(kb + NBUF - 1, nbuf);
-    compute(kb, buf);
+    __builtin_amdgcn_sched_barrier(0);  // no code motion across the phases: keeps the accumulators'
+#ifndef ESMOE_DBG_NOMFMA
+    compute(kb, buf);                   // live ranges from overlapping the copy set-up
+#else
+    acc[0][0][0] += *(const float*)(lds + buf * G::kStageBytes + lane * 4);
+#endif
+    __builtin_amdgcn_sched_barrier(0);
     // K block kb+1 must have landed (all but the newest NBUF-2 stages), and every wavefront must be
     // done reading slot `buf` before the next iteration's copies overwrite it
-    if (more) wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>(); else wait_vmcnt<0>();
+    if (!more) wait_vmcnt<0>();
+    else if (sa4) wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1)>();
+    else wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>();
     block_barrier();
     buf = buf + 1 == NBUF ? 0 : buf + 1;
     nbuf = nbuf + 1 == NBUF ? 0 : nbuf + 1;
@@ -338,7 +384,7 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 
 // Tile heights (MT * 16 rows) compiled into the persistent kernel.
 #ifndef ESMOE_VARIANTS
-#define ESMOE_VARIANTS ESMOE_CASE(1) ESMOE_CASE(2) ESMOE_CASE(4) ESMOE_CASE(8)
+#define ESMOE_VARIANTS ESMOE_CASE(1) ESMOE_CASE(2) ESMOE_CASE(4) ESMOE_CASE(8) ESMOE_CASE(12) ESMOE_CASE(16)
 #endif
 
 template <bool MX>

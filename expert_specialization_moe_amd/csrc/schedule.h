@@ -21,11 +21,11 @@
 
 namespace esmoe {
 
-// Row-tile heights are MT * 16 rows with MT in {1, 2, 4, 8, 16}; a workgroup tile
-// is (MT * 16) rows by (NT * 64) columns, NT in {1, 2, 4}.
+// Row-tile heights are MT * 16 rows with MT in {1, 2, 4, 8, 12, 16}; a workgroup tile
+// is (MT * 16) rows by 256 columns.
 struct SchedPolicy {
   int force_mt;   // 0 = choose per expert; else every tile uses this MT
-  int big_mt;     // MT of the full tiles of a many-row expert (8 or 16)
+  int big_mt;     // MT of the full tiles of a many-row expert (8, 12 or 16)
   int order;      // 0: experts sorted by rows, most rows first; 1: expert index order
 };
 
@@ -36,10 +36,16 @@ struct TileCoord {
   int n0;  // first column
 };
 
+// Smallest tile height of the menu {1, 2, 4, 8, 12, 16} (x16 rows) that covers `rows`, at most max_mt.
 ESMOE_HD int sched_cover_mt(int rows, int max_mt) {
+  const int need = (rows + 15) / 16;
   int mt = 1;
-  while (mt * 16 < rows && mt < max_mt) mt *= 2;
-  return mt;
+  if (need > 1) mt = 2;
+  if (need > 2) mt = 4;
+  if (need > 4) mt = 8;
+  if (need > 8) mt = 12;
+  if (need > 12) mt = 16;
+  return mt < max_mt ? mt : max_mt;
 }
 
 // Every compiled shape is 256 columns wide (NT = 4 units of 64).
