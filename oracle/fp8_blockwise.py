@@ -23,14 +23,16 @@ def quant_act_1x128(x):
     """[M, K] float32 (K % 128 == 0) -> (codes uint8 [M, K], scales float32 [M, K/128]).
 
     amax over each 1x128 block, clamped below at 1e-4; data = e4m3(x * (448 / amax))
-    with the product formed in fp32; scale = amax / 448.
+    with the product formed in fp32; scale = amax / 448.  The reference writes the multiplier as
+    ``448.0 / x_amax`` with a Python scalar on the left, which torch evaluates as
+    ``reciprocal(x_amax) * 448.0`` (two fp32 roundings, not one division); the same is done here.
     """
     x = np.asarray(x, dtype=np.float32)
     m, k = x.shape
     assert k % BLOCK == 0
     xv = x.reshape(m, k // BLOCK, BLOCK)
     amax = np.maximum(np.abs(xv).max(axis=2), np.float32(1e-4)).astype(np.float32)
-    mult = (np.float32(448.0) / amax).astype(np.float32)
+    mult = ((np.float32(1.0) / amax).astype(np.float32) * np.float32(448.0)).astype(np.float32)
     scaled = (xv * mult[:, :, None]).astype(np.float32)
     codes = fp8.e4m3fn_encode_rne(scaled).reshape(m, k)
     return codes, (amax / np.float32(448.0)).astype(np.float32)
@@ -48,18 +50,19 @@ def quant_weight_128x128(w):
     assert n % BLOCK == 0 and k % BLOCK == 0
     wv = w.reshape(n // BLOCK, BLOCK, k // BLOCK, BLOCK)
     amax = np.maximum(np.abs(wv).max(axis=(1, 3)), np.float32(1e-4)).astype(np.float32)
-    mult = (np.float32(448.0) / amax).astype(np.float32)
+    mult = ((np.float32(1.0) / amax).astype(np.float32) * np.float32(448.0)).astype(np.float32)
     scaled = (wv * mult[:, None, :, None]).astype(np.float32)
     codes = fp8.e4m3fn_encode_rne(scaled).reshape(n, k)
     return codes, (amax / np.float32(448.0)).astype(np.float32)
 
 
-def dequant_act(a_codes, sa):
-    return fp8.e4m3fn_decode(a_codes) * np.repeat(sa, BLOCK, axis=1)
+def dequant_act(a_codes, sa, dtype=np.float32):
+    """scale * value, formed in `dtype` (fp32 as the reference does; fp64 is exact)."""
+    return fp8.e4m3fn_decode(a_codes).astype(dtype) * np.repeat(sa, BLOCK, axis=1).astype(dtype)
 
 
-def dequant_weight(b_codes, sb):
-    return fp8.e4m3fn_decode(b_codes) * np.repeat(np.repeat(sb, BLOCK, axis=0), BLOCK, axis=1)
+def dequant_weight(b_codes, sb, dtype=np.float32):
+    return fp8.e4m3fn_decode(b_codes).astype(dtype) * np.repeat(np.repeat(sb, BLOCK, axis=0), BLOCK, axis=1).astype(dtype)
 
 
 def _round_out(y, out_dtype):
@@ -93,8 +96,8 @@ def grouped_mm(a_codes, b_codes, sa, sb, problem_sizes, expert_offsets, out_dtyp
             continue
         assert n_e == n and k_e == k
         off = int(expert_offsets[e])
-        a32 = dequant_act(a_codes[off:off + m_e], sa[off:off + m_e]).astype(dt)
-        b32 = dequant_weight(b_codes[e], sb[e]).astype(dt)
+        a32 = dequant_act(a_codes[off:off + m_e], sa[off:off + m_e], dt)
+        b32 = dequant_weight(b_codes[e], sb[e], dt)
         y = _matmul_nt(a32, b32)
         out[off:off + m_e] = _round_out(y, out_dtype)
     return out

@@ -1,0 +1,157 @@
+"""GPU checks that do not need the oracle at full size: exact special cases, untouched rows,
+size-independent properties at the benchmark configurations' real shapes."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8
+from oracle import fp8_blockwise as ofp8
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _int_operands(rows, n, k, seed, dev="cuda"):
+    """Small-integer fp8 operands with unit scales: the GEMM result is an exact integer matmul."""
+    from expert_specialization_moe_amd import workloads as W
+
+    rng = np.random.default_rng(seed)
+    e, total = len(rows), sum(rows)
+    ai = rng.integers(-3, 4, size=(total, k)).astype(np.float32)
+    bi = rng.integers(-3, 4, size=(e, n, k)).astype(np.float32)
+    ops = {
+        "a": torch.from_numpy(fp8.e4m3fn_encode_rne(ai)).to(dev).view(torch.float8_e4m3fn),
+        "b_phys": torch.from_numpy(fp8.e4m3fn_encode_rne(bi)).to(dev).view(torch.float8_e4m3fn),
+        "scales_a": torch.ones((total, k // 128), device=dev),
+        "scales_b_phys": torch.ones((e, n // 128, k // 128), device=dev),
+        "problem_sizes": torch.tensor([[m, n, k] for m in rows], dtype=torch.int32, device=dev),
+        "expert_offsets": torch.tensor(W.offsets_of(rows), dtype=torch.int32, device=dev),
+        "output": torch.full((total, n), float("nan"), dtype=torch.bfloat16, device=dev),
+    }
+    return ops, ai, bi
+
+
+@pytest.mark.parametrize("force_bm", [0, 16, 128, 192, 256])
+def test_exact_integer_gemm(esmoe, force_bm):
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import workloads as W
+
+    rows, n, k = [40, 0, 3, 200], 256, 256   # |sum| <= 9 * 256 = 2304: not all bf16-exact, so compare after rounding
+    ops, ai, bi = _int_operands(rows, n, k, seed=11)
+    y = H.f32(H.capi_fp8_mm(_native, ops, force_bm=force_bm))
+    for e, (m, off) in enumerate(zip(rows, W.offsets_of(rows))):
+        if m:
+            exact = ai[off:off + m] @ bi[e].T
+            assert np.array_equal(y[off:off + m], fp8.bf16_round(exact.astype(np.float32))), f"expert {e}"
+
+
+def test_rows_of_no_expert_are_not_written(esmoe):
+    from expert_specialization_moe_amd import _native
+
+    rows, n, k = [5, 0, 17], 128, 128
+    ops, _, _ = _int_operands(rows, n, k, seed=12)
+    # 7 spare rows after the last expert in the same buffers
+    spare = 7
+    big_out = torch.full((sum(rows) + spare, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops["a"] = torch.cat([ops["a"].view(torch.uint8), torch.zeros((spare, k), dtype=torch.uint8, device="cuda")]).view(torch.float8_e4m3fn)
+    ops["scales_a"] = torch.cat([ops["scales_a"], torch.ones((spare, k // 128), device="cuda")])
+    y = H.capi_fp8_mm(_native, ops, out=big_out)
+    assert torch.isnan(y[-spare:]).all() and not torch.isnan(y[:-spare]).any()
+
+
+def test_power_of_two_scale_shift_and_expert_permutation(esmoe):
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import workloads as W
+
+    prob = W.Problem("p", 256, 384, [70, 9, 131])
+    ops = W.make_fp8_blockwise_operands(prob, "cuda", seed=13)
+    y1 = H.capi_fp8_mm(_native, ops).clone()
+    ops2 = dict(ops, scales_a=ops["scales_a"] * 4.0, output=torch.empty_like(ops["output"]))
+    y2 = H.capi_fp8_mm(_native, ops2)
+    assert torch.equal(y2.float(), y1.float() * 4.0)
+    # experts listed in another order (same rows, same weights): identical bits per expert
+    perm = [2, 0, 1]
+    offs = W.offsets_of(prob.rows)
+    ops3 = dict(ops, b_phys=ops["b_phys"][perm].contiguous(), scales_b_phys=ops["scales_b_phys"][perm].contiguous(),
+                problem_sizes=ops["problem_sizes"][perm].contiguous(),
+                expert_offsets=torch.tensor([offs[i] for i in perm], dtype=torch.int32, device="cuda"),
+                output=torch.empty_like(ops["output"]))
+    y3 = H.capi_fp8_mm(_native, ops3)
+    assert torch.equal(y3, y1)
+
+
+@pytest.mark.parametrize("cfg", ["c1", "c2"])
+def test_benchmark_shapes_sampled_against_oracle(esmoe, cfg):
+    """Real shapes of the benchmark configurations; the oracle checks a sample of experts and columns."""
+    from expert_specialization_moe_amd import workloads as W
+
+    prob = W.config_problem(cfg, seed=0)
+    ops = W.make_fp8_blockwise_operands(prob, "cuda", seed=0)
+    ops["output"].fill_(float("nan"))
+    esmoe.es_fp8_blockwise_scaled_grouped_mm(ops["output"], ops["a"], ops["b"], ops["scales_a"], ops["scales_b"],
+                                             ops["stride_a"], ops["stride_b"], ops["stride_d"], ops["problem_sizes"],
+                                             ops["expert_offsets"], ops["workspace"])
+    torch.cuda.synchronize()
+    out = ops["output"]
+    assert not torch.isnan(out).any()
+    offs = W.offsets_of(prob.rows)
+    order = np.argsort(prob.rows)
+    picks = [int(order[-1]), int(order[len(order) // 2]), int(next(i for i in order if prob.rows[i] > 0))]
+    for e in picks:
+        m, off = prob.rows[e], int(offs[e])
+        m_s = min(m, 300)                      # first rows and last rows of the expert
+        rows_idx = np.unique(np.concatenate([np.arange(min(m_s, m)), np.arange(max(0, m - 40), m)]))
+        cols = slice(prob.n - 384, prob.n)     # last three 128-column blocks
+        a = H.codes(ops["a"][off:off + m])[rows_idx]
+        sa = H.f32(ops["scales_a"][off:off + m])[rows_idx]
+        b = H.codes(ops["b_phys"][e, cols])[None]
+        sb = H.f32(ops["scales_b_phys"][e, (prob.n - 384) // 128:])[None]
+        ref = ofp8.grouped_mm(a, b, sa, sb, [[len(rows_idx), 384, prob.k]], [0])
+        y = H.f32(out[off:off + m, cols])[rows_idx]
+        H.check_close(y, ref, f"{cfg} expert {e}")
+
+
+def test_reference_style_diff_against_unquantised_product(esmoe):
+    """The reference's own acceptance test: calc_diff(actual, a @ b) < 1e-3 per expert
+    (test/test_es_grouped_gemm.py:195-199), both output dtypes."""
+    from expert_specialization_moe_amd import quant
+
+    for out_dtype in (torch.bfloat16, torch.half):
+        gen = torch.Generator(device="cuda").manual_seed(21)
+        e, n, k = 8, 384, 640
+        rows = [int(v) for v in torch.randint(1, 257, (e,), generator=torch.Generator().manual_seed(3))]
+        total = sum(rows)
+        a = torch.randn((total, k), device="cuda", dtype=out_dtype, generator=gen)
+        w = torch.randn((e, n, k), device="cuda", dtype=out_dtype, generator=gen)
+        a_q, sa = quant.quant_act_1x128(a)
+        b_q, sb = quant.quant_weight_128x128(w)
+        offs = np.concatenate([[0], np.cumsum(rows)[:-1]])
+        ps = torch.tensor([[m, n, k] for m in rows], dtype=torch.int32, device="cuda")
+        eo = torch.tensor(offs, dtype=torch.int32, device="cuda")
+        out = torch.empty((total, n), dtype=out_dtype, device="cuda")
+        st = torch.full((e,), k, dtype=torch.int64, device="cuda")
+        esmoe.es_fp8_blockwise_scaled_grouped_mm(out, a_q.contiguous(), b_q.transpose(1, 2), sa.contiguous(),
+                                                 sb.transpose(1, 2), st, st,
+                                                 torch.full((e,), n, dtype=torch.int64, device="cuda"), ps, eo,
+                                                 torch.empty((1024,), dtype=torch.uint8, device="cuda"))
+        torch.cuda.synchronize()
+        for g, (m, off) in enumerate(zip(rows, offs)):
+            base = (a[off:off + m].float() @ w[g].float().t()).cpu().numpy()
+            assert ofp8.calc_diff(H.f32(out[off:off + m]), base) < 1e-3
+
+
+def test_small_k_and_many_experts(esmoe):
+    """K = 256 / 384 (fewer than 4 K blocks: per-block activation scales path) and 128 experts."""
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import workloads as W
+    from oracle import fp8_blockwise as o
+
+    rng = np.random.default_rng(5)
+    for k in (128, 256, 384):
+        rows = [int(v) for v in rng.integers(0, 40, size=128)]
+        prob = W.Problem("many", 256, k, rows)
+        ops = W.make_fp8_blockwise_operands(prob, "cuda", seed=k)
+        y = H.f32(H.capi_fp8_mm(_native, ops))
+        ref = o.grouped_mm(H.codes(ops["a"]), H.codes(ops["b_phys"]), H.f32(ops["scales_a"]), H.f32(ops["scales_b_phys"]),
+                           [[m, 256, k] for m in rows], W.offsets_of(rows))
+        H.check_grouped(y, ref, rows, W.offsets_of(rows), f"k={k}")
