@@ -278,7 +278,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 
   // ---- pipeline --------------------------------------------------------------------------
   // prologue: NBUF-1 K blocks in flight
-  if (sa4) issue_sa_chunk(0);
+  if (sa4 && wave * 64 < G::BM) issue_sa_chunk(0);
 #pragma unroll
   for (int s = 0; s < NBUF - 1; s++) {
     if (s < KB) issue(s, s);
@@ -298,12 +298,19 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   block_barrier();
 
   int buf = 0, nbuf = NBUF - 1;  // ring slots of K block kb and of K block kb + NBUF - 1
+  int chunk_age = NBUF;          // iterations since this wavefront issued a scale-chunk copy
   for (int kb = 0; kb < KB; kb++) {
     const bool more = kb + NBUF - 1 < KB;
-    // next chunk of activation scales, 4 K blocks before its first use: at least 3 end-of-iteration
-    // waits lie in between and each of them retires everything older than the newest NBUF-2 stages
-    if (sa4 && (kb & 3) == 0 && kb + 4 < KB) issue_sa_chunk((kb >> 2) + 1);
+    // next chunk of activation scales, 4 K blocks before its first use (only the wavefronts whose
+    // 64 rows exist in the tile fetch); `chunk_age` counts the iterations since this wavefront
+    // issued one, so that the end-of-iteration wait can leave it in flight with the newest stages
+    if (sa4 && (kb & 3) == 0 && kb + 4 < KB && wave * 64 < G::BM) {
+      issue_sa_chunk((kb >> 2) + 1);
+      chunk_age = 0;
+    }
+#if !defined(ESMOE_ISSUE_AFTER) && !defined(ESMOE_DBG_NODMA)
     if (more) issue(kb + NBUF - 1, nbuf);
+#endif
     __builtin_amdgcn_sched_barrier(0);  // no code motion across the phases: keeps the accumulators'
 #ifndef ESMOE_DBG_NOMFMA
     compute(kb, buf);                   // live ranges from overlapping the copy set-up
@@ -311,11 +318,16 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     acc[0][0][0] += *(const float*)(lds + buf * G::kStageBytes + lane * 4);
 #endif
     __builtin_amdgcn_sched_barrier(0);
+#ifdef ESMOE_ISSUE_AFTER
+    if (more) issue(kb + NBUF - 1, nbuf);
+#endif
     // K block kb+1 must have landed (all but the newest NBUF-2 stages), and every wavefront must be
     // done reading slot `buf` before the next iteration's copies overwrite it
     if (!more) wait_vmcnt<0>();
-    else if (sa4) wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1)>();
-    else wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>();
+    else if (!sa4) wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>();
+    else if (chunk_age < NBUF - 2) wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1) + 1>();
+    else wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1)>();
+    chunk_age++;
     block_barrier();
     buf = buf + 1 == NBUF ? 0 : buf + 1;
     nbuf = nbuf + 1 == NBUF ? 0 : nbuf + 1;
