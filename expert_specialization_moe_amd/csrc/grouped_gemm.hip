@@ -51,6 +51,19 @@ constexpr int kRingBytes = 148 * 1024;  // LDS ring of K-block stages
 constexpr int kMaxKB = 256;             // K <= 32768: per-tile table of weight block scales
 constexpr int kSaChunkBytes = 2 * 256 * 16;  // fp8-blockwise: two buffers of [256 rows][4 K blocks] activation scales
 constexpr int kLdsBytes = kRingBytes + 2 * kMaxKB * 4 + kSaChunkBytes;
+#ifdef ESMOE_TRACE
+constexpr int kTraceBytes = 8 * 8 * 6 * 4;
+#define ESMOE_STAMP(i)                                                                \
+  if (kb >= 16 && kb < 24) {                                                          \
+    uint64_t t_ = __builtin_amdgcn_s_memtime();                                       \
+    uint32_t v_ = (uint32_t)t_;                                                       \
+    if (lane == 0) ((uint32_t*)(lds + kLdsBytes))[(wave * 8 + (kb - 16)) * 6 + (i)] = v_; \
+    asm volatile("" ::: "memory");                                                    \
+  }
+#else
+constexpr int kTraceBytes = 0;
+#define ESMOE_STAMP(i)
+#endif
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   v8i r;
@@ -69,6 +82,26 @@ __device__ __forceinline__ void dma16(const void* base, uint32_t voff, uint32_t 
 }
 __device__ __forceinline__ void dma4(const void* base, uint32_t voff, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+// Groups of copies whose LDS destinations are 1024 bytes apart share one write of m0 and use the
+// instruction's immediate offset, which the hardware adds to the LDS address and to the global
+// address alike (so base i must already have i*1024 subtracted).  Writing m0 between two copies
+// costs a wavefront on the order of 150 cycles: the write waits until the previous copy has read it.
+__device__ __forceinline__ void dma16x2(uint32_t lds_addr, const void* b0, uint32_t v0, const void* b1, uint32_t v1) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %3, %4 offset:1024"
+               ::"s"(lds_addr), "v"(v0), "s"(b0), "v"(v1), "s"(b1) : "memory", "m0");
+}
+__device__ __forceinline__ void dma16x3(uint32_t lds_addr, const void* b0, uint32_t v0, const void* b1, uint32_t v1,
+                                        const void* b2, uint32_t v2) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %3, %4 offset:1024\n\t"
+               "global_load_lds_dwordx4 %5, %6 offset:2048"
+               ::"s"(lds_addr), "v"(v0), "s"(b0), "v"(v1), "s"(b1), "v"(v2), "s"(b2) : "memory", "m0");
+}
+__device__ __forceinline__ void dma16x4(uint32_t lds_addr, const void* b0, uint32_t v0, const void* b1, uint32_t v1,
+                                        const void* b2, uint32_t v2, const void* b3, uint32_t v3) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %3, %4 offset:1024\n\t"
+               "global_load_lds_dwordx4 %5, %6 offset:2048\n\tglobal_load_lds_dwordx4 %7, %8 offset:3072"
+               ::"s"(lds_addr), "v"(v0), "s"(b0), "v"(v1), "s"(b1), "v"(v2), "s"(b2), "v"(v3), "s"(b3) : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -166,26 +199,41 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 
   // scales of K blocks 4c .. 4c+3 into chunk buffer c & 1
   auto issue_sa_chunk = [&](int c) { dma16(sc_base + (long)c * 16, scoff, lds0 + sclds + (c & 1) * 4096); };
-  auto issue = [&](int kb, int buf) {
+  // copies of K block kb into ring slot buf: this wavefront's token blocks (consecutive 8-row blocks
+  // wave*kACopies + i; short tiles are copied by several wavefronts), its 4 weight blocks, its share
+  // of the scales
+  const int ablk0 = (wave * G::kACopies) % G::kABlocks;
+  const bool a_interior = (ablk0 + G::kACopies) * 8 - 1 <= a_last;
+  const uint32_t ro_a0 = (ablk0 & 1) ? ro_odd : ro_even, ro_a1 = ro_a0 ^ 64u;
+  const uint32_t ro_w0 = ro_even, ro_w1 = ro_odd;   // a wavefront's first weight block is even
+  // weight block i of this wavefront, i*1024 already subtracted; blocks past the last weight row are
+  // replaced by valid ones
+  long w_off[G::kWCopies];
+#pragma unroll
+  for (int i = 0; i < G::kWCopies; i++) {
+    const int blk = wave * G::kWCopies + i;
+    const int src = n0 + blk * 8 < N ? blk : i;
+    w_off[i] = (long)src * 8 * K - i * 1024;
+  }
+  auto issue_a = [&](int kb, int buf) {
     const uint32_t sb = lds0 + buf * G::kStageBytes;
     const uint8_t* ab = a_base + (long)kb * 128;
-    const uint8_t* wb = w_base + (long)kb * 128;
+    if (a_interior) {
+      const uint8_t* a0 = ab + (long)ablk0 * 8 * K;
+      const uint32_t la = sb + ablk0 * 1024;
+      const long st = 8L * K - 1024;
+      if constexpr (G::kACopies == 1) dma16(a0, ro_a0, la);
+      else if constexpr (G::kACopies == 2) dma16x2(la, a0, ro_a0, a0 + st, ro_a1);
+      else if constexpr (G::kACopies == 3) dma16x3(la, a0, ro_a0, a0 + st, ro_a1, a0 + 2 * st, ro_a0);
+      else dma16x4(la, a0, ro_a0, a0 + st, ro_a1, a0 + 2 * st, ro_a0, a0 + 3 * st, ro_a1);
+    } else {
 #pragma unroll
-    for (int i = 0; i < G::kACopies; i++) {
-      const int blk = (wave + kWaves * i) % G::kABlocks;   // short tiles are copied by several wavefronts
-      if (blk * 8 + 7 <= a_last) {
-        dma16(ab + (long)blk * 8 * K, (blk & 1) ? ro_odd : ro_even, sb + blk * 1024);
-      } else {
+      for (int i = 0; i < G::kACopies; i++) {
+        const int blk = ablk0 + i;
         int row = blk * 8 + crow;
         int grow = row > a_last ? a_last : row;
         dma16(ab, (uint32_t)grow * (uint32_t)K + (swz(row, cslot) << 4), sb + blk * 1024);
       }
-    }
-#pragma unroll
-    for (int i = 0; i < G::kWCopies; i++) {
-      const int blk = wave * G::kWCopies + i;
-      const int src = n0 + blk * 8 < N ? blk : i;          // past the last weight row: copy valid rows instead
-      dma16(wb + (long)src * 8 * K, (blk & 1) ? ro_odd : ro_even, sb + G::kABytes + blk * 1024);
     }
     if constexpr (!MX) {
       if (!sa4) dma4(sc_base + (long)kb * 4, scoff, sb + sclds);
@@ -193,6 +241,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       dma16(sc_base + (long)kb * 512, scoff, sb + sclds);
     }
   };
+  auto issue_w = [&](int kb, int buf) {
+    const uint32_t sb = lds0 + buf * G::kStageBytes;
+    const uint8_t* wb = w_base + (long)kb * 128;
+    static_assert(G::kWCopies == 4, "weight copies per wavefront");
+    dma16x4(sb + G::kABytes + wave * G::kWCopies * 1024, wb + w_off[0], ro_w0, wb + w_off[1], ro_w1, wb + w_off[2], ro_w0,
+            wb + w_off[3], ro_w1);
+  };
+  auto issue = [&](int kb, int buf) { issue_a(kb, buf); issue_w(kb, buf); };
 
   // ---- fragment read plan ----------------------------------------------------------------
   // token fragment of row tile mt: LDS row ra = mw + mt*16 + r, chunks gq and gq+4
@@ -214,15 +270,30 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
     for (int mt = 0; mt < MTW; mt++) acc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  auto compute = [&](int kb, int buf) {
-    const uint8_t* lb = lds + buf * G::kStageBytes;
+  // The work on one K block is split in two phases, so that the two groups of four wavefronts (one
+  // wavefront of each group per SIMD) can run half an iteration apart: while one group's MFMAs keep
+  // the matrix pipe busy, the other group reads its fragments from LDS.
+  //   read phase: weight fragments, the first kPre token fragments and all scales -> registers
+  //   mfma phase: the MFMAs (+ the fp32 promotion for fp8-blockwise) of the K block
+  constexpr int kPre = MTW < 4 ? MTW : (MTW == 6 ? 6 : 4);
+  struct Frags {
     v8i wf[NTW];
+    v8i af[kPre];
+    int sfw[MX ? NTW : 1];
+    int sfa[MX ? MTW : 1];
+    float sc[MX ? 1 : MTW];
+  };
+
+  auto read_phase = [&](int kb, int buf, Frags& f) {
+    const uint8_t* lb = lds + buf * G::kStageBytes;
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
-      wf[nt] = join(*(const v4i*)(lb + wfrag_lo + nt * 2048), *(const v4i*)(lb + (wfrag_lo ^ 64) + nt * 2048));
+      f.wf[nt] = join(*(const v4i*)(lb + wfrag_lo + nt * 2048), *(const v4i*)(lb + (wfrag_lo ^ 64) + nt * 2048));
     }
-    int sfw[MX ? NTW : 1];
-    float sbv = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < kPre; mt++) {
+      f.af[mt] = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + (afrag_lo ^ 64) + mt * 2048));
+    }
     if constexpr (MX) {
       // scale dword of weight row nl = nw + nt*16 + r inside the swizzled 512-byte tiles: nw is a
       // multiple of NTW*16, so the tile / quarter / row parts of nt are compile-time offsets
@@ -230,28 +301,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       for (int nt = 0; nt < NTW; nt++) {
         constexpr int kQuarter = NTW == 4 ? 1 : 0;  // NTW = 4: nt/2 selects the 32-row quarter
         uint32_t d = *(const uint32_t*)(lb + sfw_lane + (nt & 1) * 256 + (kQuarter ? (nt >> 1) * 4 : 0));
-        sfw[nt] = (int)(d >> (gq * 8));
+        f.sfw[nt] = (int)(d >> (gq * 8));
       }
-    } else {
-      sbv = sb_tab[kb];
-    }
 #pragma unroll
-    for (int mt = 0; mt < MTW; mt++) {
-      v8i afr = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + (afrag_lo ^ 64) + mt * 2048));
-      if constexpr (!MX) {
-        float sc = (sa4 ? *(const float*)(lds + sa4_lane + ((kb >> 2) & 1) * 4096 + (kb & 3) * 4 + mt * 256)
-                        : *(const float*)(lb + sa_lane + mt * 64)) * sbv;
-        v4f tmp[NTW];
-#pragma unroll
-        for (int nt = 0; nt < NTW; nt++) {
-          tmp[nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], afr, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-        }
-#pragma unroll
-        for (int nt = 0; nt < NTW; nt++) {
-#pragma unroll
-          for (int i = 0; i < 4; i++) acc[nt][mt][i] = __builtin_fmaf(tmp[nt][i], sc, acc[nt][mt][i]);
-        }
-      } else {
+      for (int mt = 0; mt < MTW; mt++) {
         uint32_t d;
         if constexpr (MT == 8 || MT == 16) {
           // tall tiles start on a 128-row boundary and a wavefront's rows start on a multiple of its
@@ -264,16 +317,80 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
           int ml = (m0 & 127) + mt * 16 + r;  // token row inside its 128-row scale tile
           d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml & 31) * 16 + (ml >> 5) * 4);
         }
-        int sfa = (int)(d >> (gq * 8));
+        f.sfa[mt] = (int)(d >> (gq * 8));
+      }
+    } else {
+      const float sbv = sb_tab[kb];
+#pragma unroll
+      for (int mt = 0; mt < MTW; mt++) {
+        f.sc[mt] = (sa4 ? *(const float*)(lds + sa4_lane + ((kb >> 2) & 1) * 4096 + (kb & 3) * 4 + mt * 256)
+                        : *(const float*)(lb + sa_lane + mt * 64)) * sbv;
+      }
+    }
+  };
+
+  // The fp32 promotion of row tile mt runs behind the MFMAs of row tile mt + 1, so that the vector ALU
+  // works in the shadow of the matrix pipe.
+  auto mfma_phase = [&](int buf, const Frags& f) {
+    const uint8_t* lb = lds + buf * G::kStageBytes;
+#ifdef ESMOE_DBG_NOMFMA
+    {
+      int x = 0;
+      for (int nt = 0; nt < NTW; nt++) for (int j = 0; j < 8; j++) x ^= f.wf[nt][j];
+      for (int mt = 0; mt < kPre; mt++) for (int j = 0; j < 8; j++) x ^= f.af[mt][j];
+      acc[0][0][0] += __builtin_bit_cast(float, x & 0x3fffffff);
+      return;
+    }
+#endif
+    v4f tmp[2][NTW];
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) {
+      v8i afr;
+      if (mt < kPre) afr = f.af[mt < kPre ? mt : 0];
+      else afr = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + (afrag_lo ^ 64) + mt * 2048));
+      if constexpr (!MX) {
+#ifdef ESMOE_DBG_NOFMA
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++) {
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nt], afr, acc[nt][mt], 0, 0, 0, sfw[nt], 0, sfa);
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], afr, acc[nt][mt], 0, 0, 0, 0, 0, 0);
+        }
+#else
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) {
+          tmp[mt & 1][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], afr, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+        }
+#endif
+      } else {
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) {
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], afr, acc[nt][mt], 0, 0, 0, f.sfw[nt], 0, f.sfa[mt]);
         }
       }
-#ifdef ESMOE_MT_SCHED_BARRIER
-      if constexpr (MTW >= 8) __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_sched_barrier(0);
+#ifndef ESMOE_DBG_NOFMA
+      if constexpr (!MX) {
+        if (mt > 0) {
+#pragma unroll
+          for (int nt = 0; nt < NTW; nt++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[nt][mt - 1][i] = __builtin_fmaf(tmp[(mt - 1) & 1][nt][i], f.sc[mt - 1], acc[nt][mt - 1][i]);
+            asm volatile("" : "+v"(acc[nt][mt - 1]));  // keeps the promotion here, in the shadow of the MFMAs above
+          }
+        }
+      }
 #endif
+      __builtin_amdgcn_sched_barrier(0);
     }
+#ifndef ESMOE_DBG_NOFMA
+    if constexpr (!MX) {
+#pragma unroll
+      for (int nt = 0; nt < NTW; nt++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[nt][MTW - 1][i] = __builtin_fmaf(tmp[(MTW - 1) & 1][nt][i], f.sc[MTW - 1], acc[nt][MTW - 1][i]);
+        asm volatile("" : "+v"(acc[nt][MTW - 1]));
+      }
+    }
+#endif
   };
 
   // ---- pipeline --------------------------------------------------------------------------
@@ -297,42 +414,91 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   else wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>();
   block_barrier();
 
+  // Barrier intervals alternate; group 0 (wavefronts 0-3) reads K block kb in interval 2kb and runs its
+  // MFMAs in interval 2kb+1, group 1 (wavefronts 4-7) does each one interval later.  Ring slot of K
+  // block kb is therefore read during intervals 2kb and 2kb+1 and must be complete before interval
+  // 2kb starts; it is refilled with K block kb+NBUF from interval 2kb+2 on: by group 1 at the start of
+  // its mfma phase kb (interval 2kb+2), by group 0 at the start of its mfma phase kb+1 (interval 2kb+3).
+  // Issuing the copies costs a wavefront a few hundred cycles; putting them in front of the MFMAs
+  // evens out the two groups' phases (the read phase waits on LDS latency already).
+  // Tiles whose mfma phase still reads token fragments from LDS (16 row tiles per wavefront do not
+  // fit in registers) run both groups in step, with no barrier between the phases.
+  constexpr bool kPP = kPre == MTW;
+#ifndef ESMOE_PP_GRP
+#define ESMOE_PP_GRP 0
+#endif
+  const int grp = !kPP ? 0 : ESMOE_PP_GRP == 0 ? wave >> 2 : ESMOE_PP_GRP == 1 ? wave & 1 : (wave >> 1) & 1;
+  auto wait_stage = [&](bool more, int chunk_young) {
+    // all of this wavefront's copies except those of the newest NBUF-2 K blocks have landed
+    if (!more) wait_vmcnt<0>();
+    else if (!sa4) wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>();
+    else if (chunk_young) wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1) + 1>();
+    else wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1)>();
+  };
   int buf = 0, nbuf = NBUF - 1;  // ring slots of K block kb and of K block kb + NBUF - 1
   int chunk_age = NBUF;          // iterations since this wavefront issued a scale-chunk copy
+  if (grp == 1) {
+#ifndef ESMOE_DBG_NODMA
+    if (NBUF - 1 < KB) issue_w(NBUF - 1, nbuf);
+#endif
+#ifndef ESMOE_DBG_NOBAR
+    block_barrier();
+#endif
+  }
+  Frags f;
   for (int kb = 0; kb < KB; kb++) {
     const bool more = kb + NBUF - 1 < KB;
+    ESMOE_STAMP(0)
+#ifndef ESMOE_DBG_NODMA
     // next chunk of activation scales, 4 K blocks before its first use (only the wavefronts whose
-    // 64 rows exist in the tile fetch); `chunk_age` counts the iterations since this wavefront
-    // issued one, so that the end-of-iteration wait can leave it in flight with the newest stages
+    // 64 rows exist in the tile fetch); `chunk_age` counts the iterations since, so that the wait
+    // below can leave it in flight with the newest stages
     if (sa4 && (kb & 3) == 0 && kb + 4 < KB && wave * 64 < G::BM) {
       issue_sa_chunk((kb >> 2) + 1);
       chunk_age = 0;
     }
-#if !defined(ESMOE_ISSUE_AFTER) && !defined(ESMOE_DBG_NODMA)
-    if (more) issue(kb + NBUF - 1, nbuf);
-#endif
-    __builtin_amdgcn_sched_barrier(0);  // no code motion across the phases: keeps the accumulators'
-#ifndef ESMOE_DBG_NOMFMA
-    compute(kb, buf);                   // live ranges from overlapping the copy set-up
-#else
-    acc[0][0][0] += *(const float*)(lds + buf * G::kStageBytes + lane * 4);
+    if (more) { if constexpr (kPP) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
 #endif
     __builtin_amdgcn_sched_barrier(0);
-#ifdef ESMOE_ISSUE_AFTER
-    if (more) issue(kb + NBUF - 1, nbuf);
+    ESMOE_STAMP(1)
+#ifdef ESMOE_DBG_NOREAD
+    if (kb == 0) read_phase(kb, buf, f);
+#else
+    read_phase(kb, buf, f);
 #endif
-    // K block kb+1 must have landed (all but the newest NBUF-2 stages), and every wavefront must be
-    // done reading slot `buf` before the next iteration's copies overwrite it
-    if (!more) wait_vmcnt<0>();
-    else if (!sa4) wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>();
-    else if (chunk_age < NBUF - 2) wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1) + 1>();
-    else wait_vmcnt<(NBUF - 2) * (G::kCopiesPerStage - 1)>();
+    __builtin_amdgcn_sched_barrier(0);
+    ESMOE_STAMP(2)
+    if (grp == 1) wait_stage(more, chunk_age < NBUF - 2);
+#ifndef ESMOE_DBG_NOBAR
+    if constexpr (kPP) block_barrier();
+#endif
+    ESMOE_STAMP(3)
+#ifndef ESMOE_DBG_NODMA
+    if constexpr (kPP) {
+      if (grp == 0) { if (more) issue_w(kb + NBUF - 1, nbuf); }
+      else if (kb + NBUF < KB) issue_w(kb + NBUF, buf);
+    }
+#endif
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_phase(buf, f);
+    __builtin_amdgcn_sched_barrier(0);
+    ESMOE_STAMP(4)
+    if (grp == 0) wait_stage(more, chunk_age < NBUF - 2);
+    ESMOE_STAMP(5)
     chunk_age++;
+#ifndef ESMOE_DBG_NOBAR
     block_barrier();
+#endif
     buf = buf + 1 == NBUF ? 0 : buf + 1;
     nbuf = nbuf + 1 == NBUF ? 0 : nbuf + 1;
   }
+#ifndef ESMOE_DBG_NOBAR
+  if (kPP && grp == 0) block_barrier();
+#endif
 
+#ifdef ESMOE_TRACE
+  if (blockIdx.x == 0) return;
+#endif
   // epilogue: lane holds columns n0 + nw + nt*16 + 4*gq + [0,4) of token row m0 + mw + mt*16 + r
   if (wave_active) {
 #pragma unroll
@@ -401,7 +567,7 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 
 template <bool MX>
 __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes + kTraceBytes];
   __shared__ int s_item;
   int* ws = g.ws;
   const int total = ws[kWsTotal];
@@ -431,6 +597,10 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     }
 #undef ESMOE_CASE
   }
+#ifdef ESMOE_TRACE
+  __syncthreads();
+  if (blockIdx.x == 0 && threadIdx.x < kTraceBytes / 4) ((uint32_t*)g.out)[threadIdx.x] = ((const uint32_t*)(lds + kLdsBytes))[threadIdx.x];
+#endif
 }
 
 }  // namespace esmoe
