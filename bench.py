@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the expert-specialized grouped GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4] [--force-bm 0|16|...]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4] [--op gemm|quant] [--force-bm 0|16|...]
 
 One "step" is one call of the operator (through torch.ops.expert_specialization.*) over one batch
 of synthetic, already-quantised operands resident in HBM.  Prints ONE JSON line.  The default
@@ -16,6 +16,19 @@ import time
 
 import torch
 
+# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
+# this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
+# Keyed by (config, op); None where not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def calibration_copy():
+    src = torch.empty((1 << 30,), dtype=torch.uint8, device="cuda:0").fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -26,8 +39,13 @@ def parse():
     ap.add_argument("--tokens", type=int, default=8192, help="c3 only")
     ap.add_argument("--routing", default="zipf", choices=["zipf", "uniform"], help="c3 only")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--op", default="gemm", choices=["gemm", "quant"],
+                    help="quant: the MXFP8 grouped quantisation of the workload's activation rows (c4 stage 1)")
     ap.add_argument("--force-bm", type=int, default=0, help="single M-tile shape for every expert (0 = device schedule)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="after the timed region also run three 1 GiB device copies (a kernel of known traffic, for "
+                         "scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline sample")
     return ap.parse_args()
 
@@ -49,7 +67,9 @@ def cpu_baseline(prob, ops, budget_s):
     used = 0.0
     done = 0
     a_codes = ops["a"].contiguous().view(torch.uint8).cpu().numpy()
-    for e, m in enumerate(rows):
+    order = [e for _ in range(64) for e in range(len(rows))]   # whole passes over the experts until the budget is used
+    for e in order:
+        m = rows[e]
         if m == 0:
             done += 1
             continue
@@ -75,8 +95,71 @@ def cpu_baseline(prob, ops, budget_s):
             break
     return {
         "value": flops / used / 1e12 if used else 0.0, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-        "sample": f"first {done} of {len(rows)} experts of the same workload ({flops / 1e9:.1f} GFLOP, {used:.1f} s)",
+        "sample": f"{done} expert problems of the same workload in index order, {done / len(rows):.2f} passes "
+                  f"({flops / 1e9:.1f} GFLOP, {used:.1f} s)",
     }
+
+
+def bench_quant(args, prob, es, W):
+    """MXFP8 grouped quantisation (bf16 rows -> e4m3 bytes + swizzled E8M0 scales) of the workload's rows."""
+    import numpy as np
+
+    dev = "cuda:0"
+    rows, k, total = prob.rows, prob.k, prob.total_rows
+    gen = torch.Generator().manual_seed(args.seed)
+    x = torch.randn((total, k), generator=gen).to(torch.bfloat16)
+    xd = x.to(dev)
+    ps = torch.tensor([[m, prob.n, k] for m in rows], dtype=torch.int32, device=dev)
+    eo = torch.tensor(W.offsets_of(rows), dtype=torch.int32, device=dev)
+    bso_np, sf_rows = W.blockscale_offsets_of(rows)
+    bso = torch.tensor(bso_np, dtype=torch.int32, device=dev)
+    q = torch.empty((total, k), dtype=torch.uint8, device=dev)
+    sf = torch.zeros((sf_rows * (k // 32),), dtype=torch.uint8, device=dev)
+
+    def step():
+        es.es_sm100_mxfp8_blockscaled_grouped_quant(xd, ps, eo, bso, q, sf)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    ms_per_step = start.elapsed_time(stop) / args.steps
+    nbytes = W.quant_bytes(rows, k)
+    t = ms_per_step * 1e-3
+    roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": W.HBM_BYTES_PER_S / 1e9, "unit": "GB/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((prob.name, "quant"))
+    roof["algorithmic_bytes"] = nbytes
+    roof["roofline_us"] = nbytes / W.HBM_BYTES_PER_S * 1e6
+    out = {
+        "metric": "MXFP8 grouped quantisation, algorithmic GB/s (bf16 in, e4m3 + E8M0 out)",
+        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 -> fp8_e4m3 + e8m0", "data": "synthetic",
+        "config": {"workload": f"{prob.name} quant: E={len(rows)} K={k} rows={total} max_rows={max(rows)} seed={args.seed}"},
+        "roofline": roof,
+    }
+    if args.calibration_copy:
+        calibration_copy()
+    if not args.no_cpu_baseline:
+        from oracle import mxfp8 as omx
+
+        xs = x[: min(total, 512)].float().numpy()   # bounded sample: the first rows, repeated until the budget is used
+        used, nrows = 0.0, 0
+        while used < args.cpu_seconds:
+            t0 = time.perf_counter()
+            omx.quant_rows(xs)
+            used += time.perf_counter() - t0
+            nrows += xs.shape[0]
+        out["cpu_baseline"] = {"value": W.quant_bytes([nrows], k) / used / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"{nrows} rows of the same input through the numpy oracle ({used:.1f} s)"}
+    print(json.dumps(out), flush=True)
 
 
 def main():
@@ -94,6 +177,9 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
     prob = W.config_problem(args.config, seed=args.seed, tokens=args.tokens, routing=args.routing)
+    if args.op == "quant":
+        bench_quant(args, prob, es, W)
+        return
     mx = prob.kind == "mxfp8"
     ops = (W.make_mxfp8_operands if mx else W.make_fp8_blockwise_operands)(prob, dev, seed=args.seed)
     lib = _native.lib
@@ -155,7 +241,7 @@ def main():
     else:
         roof = {"bound": "mfma", "achieved": flops / t / 1e12, "peak": W.FP8_FLOPS_PER_S / 1e12, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((prob.name, "gemm")) if not args.force_bm else None
     roof["algorithmic_bytes"] = nbytes
     roof["roofline_us"] = t_roof * 1e6
     out = {
@@ -168,6 +254,8 @@ def main():
                    "force_bm": args.force_bm, "routing_meta": prob.meta},
         "roofline": roof, "wall_ms_per_step": wall * 1e3 / args.steps,
     }
+    if args.calibration_copy:
+        calibration_copy()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(prob, ops, args.cpu_seconds)
     print(json.dumps(out), flush=True)

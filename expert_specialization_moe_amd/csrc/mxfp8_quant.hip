@@ -47,7 +47,7 @@ __device__ __forceinline__ int mx_scale_code(float amax) {
 }
 
 template <bool FP16>
-__global__ void __launch_bounds__(kQuantThreads) mxfp8_quant_kernel(const uint16_t* __restrict__ in,
+__global__ void __launch_bounds__(kQuantThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) mxfp8_quant_kernel(const uint16_t* __restrict__ in,
                                                                     const int* __restrict__ problem_sizes,
                                                                     const int* __restrict__ expert_offsets,
                                                                     const int* __restrict__ blockscale_offsets,
