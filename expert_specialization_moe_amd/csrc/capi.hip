@@ -67,10 +67,10 @@ int env_int(const char* name, int dflt) {
 esmoe::SchedPolicy make_policy(int force_bm, int mx) {
   esmoe::SchedPolicy p;
   p.force_mt = force_bm / 16;
-  // 256-row tiles need 128 accumulator registers per lane, which the mxfp8 kernel can afford (it
-  // accumulates inside the MFMA); the fp8-blockwise kernel also needs VALU temporaries for its
-  // scale-and-accumulate step and is fastest with 128-row tiles
-  p.big_mt = env_int("ESMOE_BIG_MT", mx ? 16 : 8);
+  // Taller tiles do more MFMA work per byte copied into LDS.  The mxfp8 kernel is fastest with 256-row
+  // tiles; the fp8-blockwise kernel, whose fp32 promotion shares the vector ALU, gains nothing beyond
+  // 192 rows, and shorter full tiles leave less padding in the remainder tile.
+  p.big_mt = env_int("ESMOE_BIG_MT", mx ? 16 : 12);
   p.order = env_int("ESMOE_ORDER", 0);
   return p;
 }
