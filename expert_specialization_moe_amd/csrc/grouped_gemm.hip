@@ -10,13 +10,20 @@
 // an LDS ring with global_load_lds (no staging registers, no LDS store
 // instructions).  One wavefront instruction moves 8 rows x 128 bytes: 8 consecutive
 // lanes read one row's 128 contiguous bytes, and LDS receives the 64 lanes' 16-byte
-// chunks back to back.  The ring holds 2..4 K blocks depending on the tile height,
-// so up to 3 K blocks of loads are in flight per workgroup.  LDS rows are 128 bytes
-// apart; chunk c of row r is stored in 16-byte slot c ^ ((r >> 1) & 7), which makes
-// the MFMA fragment reads (16 rows x 16 bytes per quarter-wave) bank-conflict free.
-// Loading fragments straight from global memory is ~4x slower per CU: a fragment
-// puts consecutive lanes on different rows, i.e. 64 separate 16-byte requests per
-// instruction.
+// chunks back to back.  The ring holds 2..4 K blocks depending on the tile height
+// (148 KB of the 160 KB LDS), so up to 3 K blocks of loads are in flight per
+// workgroup; with a loaded-memory latency near 2 us that ring, not the matrix pipe,
+// bounds the tall tiles.  LDS rows are 128 bytes apart; chunk c of row r is stored in
+// 16-byte slot c ^ ((r >> 1) & 7), which makes the MFMA fragment reads (16 rows x 16
+// bytes per quarter-wave) bank-conflict free.  Loading fragments straight from global
+// memory is ~4x slower per CU: a fragment puts consecutive lanes on different rows,
+// i.e. 64 separate 16-byte requests per instruction.
+//
+// K loop.  Tiles whose fragments fit in registers (up to 192 rows) split each K block
+// in a read phase (LDS -> registers) and an MFMA phase, and run the two groups of four
+// wavefronts half an iteration apart: one group's fragment reads overlap the other
+// group's MFMAs.  Copies are issued in groups that share one write of m0 and use the
+// instruction's immediate offset.
 //
 // MFMA mapping (v_mfma[_scale]_f32_16x16x128_f8f6f4, both operands e4m3):
 //   * the weight rows ride on the instruction's "A" side and the token rows on its
@@ -51,19 +58,6 @@ constexpr int kRingBytes = 148 * 1024;  // LDS ring of K-block stages
 constexpr int kMaxKB = 256;             // K <= 32768: per-tile table of weight block scales
 constexpr int kSaChunkBytes = 2 * 256 * 16;  // fp8-blockwise: two buffers of [256 rows][4 K blocks] activation scales
 constexpr int kLdsBytes = kRingBytes + 2 * kMaxKB * 4 + kSaChunkBytes;
-#ifdef ESMOE_TRACE
-constexpr int kTraceBytes = 8 * 8 * 6 * 4;
-#define ESMOE_STAMP(i)                                                                \
-  if (kb >= 16 && kb < 24) {                                                          \
-    uint64_t t_ = __builtin_amdgcn_s_memtime();                                       \
-    uint32_t v_ = (uint32_t)t_;                                                       \
-    if (lane == 0) ((uint32_t*)(lds + kLdsBytes))[(wave * 8 + (kb - 16)) * 6 + (i)] = v_; \
-    asm volatile("" ::: "memory");                                                    \
-  }
-#else
-constexpr int kTraceBytes = 0;
-#define ESMOE_STAMP(i)
-#endif
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   v8i r;
@@ -333,15 +327,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // works in the shadow of the matrix pipe.
   auto mfma_phase = [&](int buf, const Frags& f) {
     const uint8_t* lb = lds + buf * G::kStageBytes;
-#ifdef ESMOE_DBG_NOMFMA
-    {
-      int x = 0;
-      for (int nt = 0; nt < NTW; nt++) for (int j = 0; j < 8; j++) x ^= f.wf[nt][j];
-      for (int mt = 0; mt < kPre; mt++) for (int j = 0; j < 8; j++) x ^= f.af[mt][j];
-      acc[0][0][0] += __builtin_bit_cast(float, x & 0x3fffffff);
-      return;
-    }
-#endif
     v4f tmp[2][NTW];
 #pragma unroll
     for (int mt = 0; mt < MTW; mt++) {
@@ -349,17 +334,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       if (mt < kPre) afr = f.af[mt < kPre ? mt : 0];
       else afr = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + (afrag_lo ^ 64) + mt * 2048));
       if constexpr (!MX) {
-#ifdef ESMOE_DBG_NOFMA
-#pragma unroll
-        for (int nt = 0; nt < NTW; nt++) {
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], afr, acc[nt][mt], 0, 0, 0, 0, 0, 0);
-        }
-#else
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++) {
           tmp[mt & 1][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], afr, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
         }
-#endif
       } else {
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++) {
@@ -367,7 +345,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
         }
       }
       __builtin_amdgcn_sched_barrier(0);
-#ifndef ESMOE_DBG_NOFMA
       if constexpr (!MX) {
         if (mt > 0) {
 #pragma unroll
@@ -378,10 +355,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
           }
         }
       }
-#endif
       __builtin_amdgcn_sched_barrier(0);
     }
-#ifndef ESMOE_DBG_NOFMA
     if constexpr (!MX) {
 #pragma unroll
       for (int nt = 0; nt < NTW; nt++) {
@@ -390,7 +365,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
         asm volatile("" : "+v"(acc[nt][MTW - 1]));
       }
     }
-#endif
   };
 
   // ---- pipeline --------------------------------------------------------------------------
@@ -424,10 +398,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // Tiles whose mfma phase still reads token fragments from LDS (16 row tiles per wavefront do not
   // fit in registers) run both groups in step, with no barrier between the phases.
   constexpr bool kPP = kPre == MTW;
-#ifndef ESMOE_PP_GRP
-#define ESMOE_PP_GRP 0
-#endif
-  const int grp = !kPP ? 0 : ESMOE_PP_GRP == 0 ? wave >> 2 : ESMOE_PP_GRP == 1 ? wave & 1 : (wave >> 1) & 1;
+  const int grp = kPP ? wave >> 2 : 0;
   auto wait_stage = [&](bool more, int chunk_young) {
     // all of this wavefront's copies except those of the newest NBUF-2 K blocks have landed
     if (!more) wait_vmcnt<0>();
@@ -438,18 +409,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   int buf = 0, nbuf = NBUF - 1;  // ring slots of K block kb and of K block kb + NBUF - 1
   int chunk_age = NBUF;          // iterations since this wavefront issued a scale-chunk copy
   if (grp == 1) {
-#ifndef ESMOE_DBG_NODMA
     if (NBUF - 1 < KB) issue_w(NBUF - 1, nbuf);
-#endif
-#ifndef ESMOE_DBG_NOBAR
     block_barrier();
-#endif
   }
   Frags f;
   for (int kb = 0; kb < KB; kb++) {
     const bool more = kb + NBUF - 1 < KB;
-    ESMOE_STAMP(0)
-#ifndef ESMOE_DBG_NODMA
     // next chunk of activation scales, 4 K blocks before its first use (only the wavefronts whose
     // 64 rows exist in the tile fetch); `chunk_age` counts the iterations since, so that the wait
     // below can leave it in flight with the newest stages
@@ -458,47 +423,26 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       chunk_age = 0;
     }
     if (more) { if constexpr (kPP) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
-#endif
     __builtin_amdgcn_sched_barrier(0);
-    ESMOE_STAMP(1)
-#ifdef ESMOE_DBG_NOREAD
-    if (kb == 0) read_phase(kb, buf, f);
-#else
     read_phase(kb, buf, f);
-#endif
     __builtin_amdgcn_sched_barrier(0);
-    ESMOE_STAMP(2)
     if (grp == 1) wait_stage(more, chunk_age < NBUF - 2);
-#ifndef ESMOE_DBG_NOBAR
     if constexpr (kPP) block_barrier();
-#endif
-    ESMOE_STAMP(3)
-#ifndef ESMOE_DBG_NODMA
     if constexpr (kPP) {
       if (grp == 0) { if (more) issue_w(kb + NBUF - 1, nbuf); }
       else if (kb + NBUF < KB) issue_w(kb + NBUF, buf);
     }
-#endif
     __builtin_amdgcn_sched_barrier(0);
     mfma_phase(buf, f);
     __builtin_amdgcn_sched_barrier(0);
-    ESMOE_STAMP(4)
     if (grp == 0) wait_stage(more, chunk_age < NBUF - 2);
-    ESMOE_STAMP(5)
     chunk_age++;
-#ifndef ESMOE_DBG_NOBAR
     block_barrier();
-#endif
     buf = buf + 1 == NBUF ? 0 : buf + 1;
     nbuf = nbuf + 1 == NBUF ? 0 : nbuf + 1;
   }
-#ifndef ESMOE_DBG_NOBAR
   if (kPP && grp == 0) block_barrier();
-#endif
 
-#ifdef ESMOE_TRACE
-  if (blockIdx.x == 0) return;
-#endif
   // epilogue: lane holds columns n0 + nw + nt*16 + 4*gq + [0,4) of token row m0 + mw + mt*16 + r
   if (wave_active) {
 #pragma unroll
@@ -567,7 +511,7 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 
 template <bool MX>
 __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes + kTraceBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
   __shared__ int s_item;
   int* ws = g.ws;
   const int total = ws[kWsTotal];
@@ -597,10 +541,6 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     }
 #undef ESMOE_CASE
   }
-#ifdef ESMOE_TRACE
-  __syncthreads();
-  if (blockIdx.x == 0 && threadIdx.x < kTraceBytes / 4) ((uint32_t*)g.out)[threadIdx.x] = ((const uint32_t*)(lds + kLdsBytes))[threadIdx.x];
-#endif
 }
 
 }  // namespace esmoe
