@@ -479,8 +479,8 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
   __syncthreads();
   int* item_start = ws + ws_item_start(num_experts);
   int* order = ws + ws_order(num_experts);
+  int pos = e;
   if (e < num_experts) {
-    int pos = e;
     if (policy.order == 0) {
       pos = 0;
       for (int j = 0; j < num_experts; j++) {
@@ -492,15 +492,17 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
     s_items[pos] = sched_items(m, n, policy);
   }
   __syncthreads();
-  if (e == 0) {
+  if (e < num_experts) {
+    // exclusive prefix sum over schedule positions, one position per thread
     int run = 0;
-    for (int j = 0; j < num_experts; j++) {
-      item_start[j] = run;
-      run += s_items[j];
+    for (int j = 0; j < pos; j++) run += s_items[j];
+    item_start[pos] = run;
+    if (pos == num_experts - 1) {
+      run += s_items[pos];
+      item_start[num_experts] = run;
+      ws[kWsTotal] = run;
+      ws[kWsCounter] = 0;
     }
-    item_start[num_experts] = run;
-    ws[kWsTotal] = run;
-    ws[kWsCounter] = 0;
   }
 }
 
@@ -547,7 +549,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
 
 extern "C" int esmoe_launch_grouped_gemm(const esmoe::GemmArgs* args, int mx, int grid, hipStream_t stream) {
   using namespace esmoe;
-  hipLaunchKernelGGL(schedule_kernel, dim3(1), dim3(1024), 0, stream, args->problem_sizes, args->num_experts, args->n,
+  hipLaunchKernelGGL(schedule_kernel, dim3(1), dim3((args->num_experts + 63) & ~63), 0, stream, args->problem_sizes, args->num_experts, args->n,
                      args->policy, args->ws);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return (int)err;
