@@ -19,7 +19,10 @@ import torch
 # HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    ("c1", "gemm"): 1.638e9,     # FETCH 773,495.5 x 2.000 KiB + WRITE 52,929.4 x 1.000 KiB
+    ("c4", "quant"): 1.786e8,    # FETCH 57,398.6 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
+}
 
 
 def calibration_copy():
