@@ -42,8 +42,9 @@ def parse():
     ap.add_argument("--tokens", type=int, default=8192, help="c3 only")
     ap.add_argument("--routing", default="zipf", choices=["zipf", "uniform"], help="c3 only")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--op", default="gemm", choices=["gemm", "quant"],
-                    help="quant: the MXFP8 grouped quantisation of the workload's activation rows (c4 stage 1)")
+    ap.add_argument("--op", default="gemm", choices=["gemm", "quant", "quant_act"],
+                    help="quant: the MXFP8 grouped quantisation of the workload's activation rows (c4 stage 1); "
+                         "quant_act: the FP8 1x128 activation quantisation of the same rows")
     ap.add_argument("--force-bm", type=int, default=0, help="single M-tile shape for every expert (0 = device schedule)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -104,8 +105,11 @@ def cpu_baseline(prob, ops, budget_s):
 
 
 def bench_quant(args, prob, es, W):
-    """MXFP8 grouped quantisation (bf16 rows -> e4m3 bytes + swizzled E8M0 scales) of the workload's rows."""
+    """MXFP8 grouped quantisation (bf16 rows -> e4m3 bytes + swizzled E8M0 scales) of the workload's rows, or
+    (--op quant_act) their FP8 1x128 quantisation (e4m3 bytes + fp32 scale per 128-wide block)."""
     import numpy as np
+
+    act = args.op == "quant_act"
 
     dev = "cuda:0"
     rows, k, total = prob.rows, prob.k, prob.total_rows
@@ -119,8 +123,13 @@ def bench_quant(args, prob, es, W):
     q = torch.empty((total, k), dtype=torch.uint8, device=dev)
     sf = torch.zeros((sf_rows * (k // 32),), dtype=torch.uint8, device=dev)
 
+    sc = torch.empty((total, k // 128), dtype=torch.float32, device=dev)
+
     def step():
-        es.es_sm100_mxfp8_blockscaled_grouped_quant(xd, ps, eo, bso, q, sf)
+        if act:
+            es.es_fp8_quant_act_1x128(xd, q, sc)
+        else:
+            es.es_sm100_mxfp8_blockscaled_grouped_quant(xd, ps, eo, bso, q, sf)
 
     for _ in range(args.warmup):
         step()
@@ -133,34 +142,36 @@ def bench_quant(args, prob, es, W):
     stop.record()
     torch.cuda.synchronize()
     ms_per_step = start.elapsed_time(stop) / args.steps
-    nbytes = W.quant_bytes(rows, k)
+    nbytes = float(total) * k * (2 + 1 + 4 / 128.0) if act else W.quant_bytes(rows, k)
     t = ms_per_step * 1e-3
     roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": W.HBM_BYTES_PER_S / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((prob.name, "quant"))
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((prob.name, args.op))
     roof["algorithmic_bytes"] = nbytes
     roof["roofline_us"] = nbytes / W.HBM_BYTES_PER_S * 1e6
     out = {
-        "metric": "MXFP8 grouped quantisation, algorithmic GB/s (bf16 in, e4m3 + E8M0 out)",
+        "metric": ("FP8 1x128 activation quantisation, algorithmic GB/s (bf16 in, e4m3 + fp32 scales out)" if act else
+                   "MXFP8 grouped quantisation, algorithmic GB/s (bf16 in, e4m3 + E8M0 out)"),
         "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 -> fp8_e4m3 + e8m0", "data": "synthetic",
-        "config": {"workload": f"{prob.name} quant: E={len(rows)} K={k} rows={total} max_rows={max(rows)} seed={args.seed}"},
+        "dtype": "bf16 -> fp8_e4m3 + fp32 scales" if act else "bf16 -> fp8_e4m3 + e8m0", "data": "synthetic",
+        "config": {"workload": f"{prob.name} {args.op}: E={len(rows)} K={k} rows={total} max_rows={max(rows)} seed={args.seed}"},
         "roofline": roof,
     }
     if args.calibration_copy:
         calibration_copy()
     if not args.no_cpu_baseline:
+        from oracle import fp8_blockwise as ofp8
         from oracle import mxfp8 as omx
 
         xs = x[: min(total, 512)].float().numpy()   # bounded sample: the first rows, repeated until the budget is used
         used, nrows = 0.0, 0
         while used < args.cpu_seconds:
             t0 = time.perf_counter()
-            omx.quant_rows(xs)
+            ofp8.quant_act_1x128(xs) if act else omx.quant_rows(xs)
             used += time.perf_counter() - t0
             nrows += xs.shape[0]
-        out["cpu_baseline"] = {"value": W.quant_bytes([nrows], k) / used / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        out["cpu_baseline"] = {"value": nbytes / total * nrows / used / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": f"{nrows} rows of the same input through the numpy oracle ({used:.1f} s)"}
     print(json.dumps(out), flush=True)
 
@@ -180,7 +191,7 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
     prob = W.config_problem(args.config, seed=args.seed, tokens=args.tokens, routing=args.routing)
-    if args.op == "quant":
+    if args.op != "gemm":
         bench_quant(args, prob, es, W)
         return
     mx = prob.kind == "mxfp8"

@@ -12,10 +12,12 @@ from .ops import (  # noqa: F401
     es_fp8_blockwise_scaled_grouped_mm,
     es_sm100_mxfp8_blockscaled_grouped_mm,
     es_sm100_mxfp8_blockscaled_grouped_quant,
+    es_fp8_quant_act_1x128,
 )
 
 __all__ = [
     "es_fp8_blockwise_scaled_grouped_mm",
     "es_sm100_mxfp8_blockscaled_grouped_mm",
     "es_sm100_mxfp8_blockscaled_grouped_quant",
+    "es_fp8_quant_act_1x128",
 ]

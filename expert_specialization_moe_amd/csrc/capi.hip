@@ -18,6 +18,9 @@ extern "C" int esmoe_launch_mxfp8_quant(const void* in, int in_dtype, const int*
                                         const int* expert_offsets, const int* blockscale_offsets, void* q, uint8_t* sf,
                                         int num_experts, int sf_rows, int k, hipStream_t stream);
 
+extern "C" int esmoe_launch_fp8_quant_act(const void* in, int in_dtype, void* q, float* scales, long total_rows, int k,
+                                          hipStream_t stream);
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -179,6 +182,26 @@ int esmoe_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* probl
   if (rc) return rc;
   rc = esmoe_launch_mxfp8_quant(in, in_dtype, problem_sizes, expert_offsets, blockscale_offsets, q, sf, num_experts,
                                 sf_rows, k, (hipStream_t)stream);
+  if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return 0;
+}
+
+int esmoe_fp8_quant_act_1x128(const void* in, int in_dtype, void* q, float* scales, long total_rows, int k, void* stream) {
+  g_err[0] = 0;
+  if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must align to 128, got %d", k);
+  if (in_dtype != ESMOE_IN_BF16 && in_dtype != ESMOE_IN_FP16)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in_dtype must be ESMOE_IN_BF16 or ESMOE_IN_FP16");
+  if (total_rows < 0 || total_rows > (1L << 40) / k)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "total_rows out of range: %ld", total_rows);
+  if (total_rows == 0) return 0;   // empty tensors may carry null pointers
+  if (!in || !q || !scales) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if ((uintptr_t)in % 16 || (uintptr_t)q % 8 || (uintptr_t)scales % 4)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in must be 16-byte aligned, q 8-byte aligned, scales 4-byte aligned");
+  if (total_rows == 0) return 0;
+  DeviceInfo info;
+  int rc = current_device_info(&info);
+  if (rc) return rc;
+  rc = esmoe_launch_fp8_quant_act(in, in_dtype, q, scales, total_rows, k, (hipStream_t)stream);
   if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
   return 0;
 }

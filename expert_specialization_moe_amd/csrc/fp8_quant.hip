@@ -1,0 +1,93 @@
+// FP8 1x128 activation quantisation for gfx950: bf16/fp16 rows -> e4m3fn bytes + one fp32 scale
+// per 128-wide block of a row (the operand format of the FP8-blockwise grouped GEMM).
+//
+// Arithmetic follows the torch helper the reference's callers use, per_token_cast_to_fp8
+// (test/test_es_grouped_gemm.py:36-44), rounding for rounding:
+//   amax  = max(|x| over the block, 1e-4)              (fp32)
+//   mult  = fl(fl(1 / amax) * 448)                     (torch evaluates 448.0 / t as reciprocal(t) * 448)
+//   q     = e4m3fn_rne(fl(float(x) * mult))
+//   scale = fl(amax * fl(1 / 448))                     (how torch divides a GPU tensor by a Python scalar;
+//                                                       the CPU path's true division differs by one ulp
+//                                                       for some values)
+// [M, K] row-major with K % 128 == 0 makes the blocks one flat sequence: block b covers elements
+// [128 b, 128 b + 128) of input and output and owns scales[b], so the kernel is one-dimensional.
+// 16 lanes take one block (16 bytes of input each, a 256-byte coalesced segment); the block maximum
+// is reduced with four lane swaps.  Pure streaming: 2 + 1 + 4/128 bytes per element.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace esmoe {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+constexpr int kActQuantThreads = 256;
+constexpr int kActQuantUnroll = 4;   // 16-byte loads in flight per lane
+
+template <bool FP16>
+__global__ void __launch_bounds__(kActQuantThreads) __attribute__((amdgpu_waves_per_eu(6, 8)))
+fp8_quant_act_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q, float* __restrict__ scales, long chunks) {
+  // chunk c = 8 consecutive elements; 16 consecutive chunks form one 1x128 block
+  const long first = ((long)blockIdx.x * kActQuantUnroll) * kActQuantThreads + threadIdx.x;
+  v4i raw[kActQuantUnroll];
+#pragma unroll
+  for (int u = 0; u < kActQuantUnroll; u++) {
+    const long c = first + (long)u * kActQuantThreads;
+    raw[u] = v4i{0, 0, 0, 0};
+    if (c < chunks) raw[u] = __builtin_nontemporal_load((const v4i*)(in + c * 8));
+  }
+#pragma unroll
+  for (int u = 0; u < kActQuantUnroll; u++) {
+    const long c = first + (long)u * kActQuantThreads;
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t w = (uint32_t)raw[u][i];
+      if constexpr (FP16) {
+        x[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+        x[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+      } else {
+        x[2 * i] = __builtin_bit_cast(float, w << 16);
+        x[2 * i + 1] = __builtin_bit_cast(float, w & 0xffff0000u);
+      }
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) amax = __builtin_fmaxf(amax, __builtin_fabsf(x[i]));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 1));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 2));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 4));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 8));
+    amax = __builtin_fmaxf(amax, 1e-4f);
+    const float mult = (1.0f / amax) * 448.0f;   // two roundings, as torch does
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) y[i] = __builtin_amdgcn_fmed3f(x[i] * mult, -448.f, 448.f);
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], 0, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+    if (c < chunks) {
+      __builtin_nontemporal_store(v2i{w0, w1}, (v2i*)(q + c * 8));
+      if ((threadIdx.x & 15) == 0) scales[c >> 4] = amax * (1.0f / 448.0f);
+    }
+  }
+}
+
+}  // namespace esmoe
+
+extern "C" int esmoe_launch_fp8_quant_act(const void* in, int in_dtype, void* q, float* scales, long total_rows, int k,
+                                          hipStream_t stream) {
+  using namespace esmoe;
+  const long chunks = total_rows * (long)k / 8;
+  if (chunks == 0) return 0;
+  const long per_wg = (long)kActQuantThreads * kActQuantUnroll;
+  const long grid = (chunks + per_wg - 1) / per_wg;
+  if (in_dtype == 1)
+    hipLaunchKernelGGL(fp8_quant_act_kernel<true>, dim3((unsigned)grid), dim3(kActQuantThreads), 0, stream,
+                       (const uint16_t*)in, (uint8_t*)q, scales, chunks);
+  else
+    hipLaunchKernelGGL(fp8_quant_act_kernel<false>, dim3((unsigned)grid), dim3(kActQuantThreads), 0, stream,
+                       (const uint16_t*)in, (uint8_t*)q, scales, chunks);
+  return (int)hipGetLastError();
+}

@@ -213,6 +213,30 @@ void es_sm100_mxfp8_blockscaled_grouped_quant(const torch::Tensor& input, const 
   check_rc(rc, "es_sm100_mxfp8_blockscaled_grouped_quant");
 }
 
+// Extension beyond the reference's three operators: the 1x128 activation quantiser its callers run in
+// torch (per_token_cast_to_fp8, test/test_es_grouped_gemm.py:36-44), as a device operator.
+void es_fp8_quant_act_1x128(const torch::Tensor& input, torch::Tensor& quant_output, torch::Tensor& scales) {
+  TORCH_CHECK(input.dim() == 2, "input must be 2D tensor");
+  TORCH_CHECK(input.size(1) % 128 == 0, "k must align to 128");
+  TORCH_CHECK(input.scalar_type() == torch::kBFloat16 || input.scalar_type() == torch::kHalf,
+              "dtype must be kFloat16 or kBFloat16");
+  TORCH_CHECK(input.is_contiguous(), "input must be packed row major");
+  const int64_t total_rows = input.size(0), k = input.size(1);
+  TORCH_CHECK(quant_output.is_contiguous() && quant_output.element_size() == 1 && quant_output.numel() == total_rows * k,
+              "quant_output must be a contiguous 1-byte tensor of rows * k elements");
+  TORCH_CHECK(scales.is_contiguous() && scales.scalar_type() == torch::kFloat32 && scales.numel() == total_rows * (k / 128),
+              "scales must be a contiguous float32 tensor of rows * k / 128 elements");
+  require_device(input, "es_fp8_quant_act_1x128");
+  TORCH_CHECK(quant_output.device() == input.device() && scales.device() == input.device(),
+              "all tensors must be on the same device");
+  if (total_rows == 0) return;
+  c10::DeviceGuard guard(input.device());
+  int rc = esmoe_fp8_quant_act_1x128(input.data_ptr(), input.scalar_type() == torch::kBFloat16 ? ESMOE_IN_BF16 : ESMOE_IN_FP16,
+                                     quant_output.data_ptr(), scales.data_ptr<float>(), (long)total_rows, (int)k,
+                                     current_stream(input));
+  check_rc(rc, "es_fp8_quant_act_1x128");
+}
+
 TORCH_LIBRARY(expert_specialization, m) {
   m.def(
       "es_fp8_blockwise_scaled_grouped_mm(Tensor output, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, Tensor "
@@ -224,12 +248,14 @@ TORCH_LIBRARY(expert_specialization, m) {
   m.def(
       "es_sm100_mxfp8_blockscaled_grouped_quant(Tensor input, Tensor problem_sizes, Tensor expert_offsets, Tensor "
       "blockscale_offsets, Tensor quant_output, Tensor scale_factor) -> () ");
+  m.def("es_fp8_quant_act_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
   m.impl("es_fp8_blockwise_scaled_grouped_mm", &es_fp8_blockwise_scaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_mm", &es_sm100_mxfp8_blockscaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
+  m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
 }
 
 // Same functions on the CPU key: the checks run, then require_device() raises.
@@ -237,4 +263,5 @@ TORCH_LIBRARY_IMPL(expert_specialization, CPU, m) {
   m.impl("es_fp8_blockwise_scaled_grouped_mm", &es_fp8_blockwise_scaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_mm", &es_sm100_mxfp8_blockscaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
+  m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
 }

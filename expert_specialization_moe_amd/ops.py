@@ -26,3 +26,19 @@ def es_sm100_mxfp8_blockscaled_grouped_quant(input, problem_sizes, expert_offset
     """bf16/fp16 rows -> e4m3 bytes + swizzled E8M0 scales (ops.py:40-50)."""
     _ns.es_sm100_mxfp8_blockscaled_grouped_quant.default(
         input, problem_sizes, expert_offsets, blockscale_offsets, quant_output, scale_factor)
+
+
+def es_fp8_quant_act_1x128(input, quant_output=None, scales=None):
+    """bf16/fp16 [M, K] -> (e4m3fn [M, K], fp32 scales [M, K/128]) on the device.
+
+    No counterpart among the reference's operators: it is the torch helper its callers use to
+    prepare ``a`` / ``scales_a`` (per_token_cast_to_fp8, test/test_es_grouped_gemm.py:36-44),
+    reproduced bit for bit by a HIP kernel.  Allocates the outputs when they are not given.
+    """
+    m, k = input.shape
+    if quant_output is None:
+        quant_output = torch.empty((m, k), dtype=torch.float8_e4m3fn, device=input.device)
+    if scales is None:
+        scales = torch.empty((m, k // 128), dtype=torch.float32, device=input.device)
+    _ns.es_fp8_quant_act_1x128.default(input, quant_output, scales)
+    return quant_output, scales

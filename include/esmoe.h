@@ -99,6 +99,21 @@ int esmoe_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* probl
                               uint8_t* sf, int num_experts, int total_rows, int sf_rows, int k, void* stream);
 
 /*
+ * FP8 1x128 activation quantisation: bf16/fp16 rows -> e4m3fn bytes + fp32 scale per 128-wide block,
+ * the `a` / `scales_a` operands of esmoe_fp8_blockwise_grouped_mm.
+ * The reference has no operator for this step: its callers run the torch helper per_token_cast_to_fp8
+ * (test/test_es_grouped_gemm.py:36-44, again in benchmark/benchmark_es_fp8_blockwise_moe.py:18-26);
+ * this entry point reproduces that helper's arithmetic bit for bit on the device.
+ *
+ *   in [total_rows, K] bf16 or fp16 (in_dtype), K % 128 == 0;  q [total_rows, K] bytes;
+ *   scales [total_rows, K/128] fp32.   amax = max(|x|, 1e-4) per block, q = e4m3(x * (448/amax)),
+ *   scale = amax * fl(1/448) (torch's GPU evaluation of amax / 448.0).  Rows are independent, so the
+ *   grouped layout needs no metadata.
+ */
+int esmoe_fp8_quant_act_1x128(const void* in, int in_dtype, void* q, float* scales, long total_rows, int k,
+                              void* stream);
+
+/*
  * Host mirrors of the device-side tile schedule, for inspection and CPU tests; they touch no GPU.
  * No counterpart in the reference (its schedule lives inside CUTLASS's grouped tile scheduler).
  * esmoe_host_schedule fills `ws_host` (esmoe_gemm_workspace_bytes(E) bytes of host memory) from host

@@ -19,13 +19,16 @@ from . import fp8
 BLOCK = 128
 
 
-def quant_act_1x128(x):
+def quant_act_1x128(x, scale_via_reciprocal=False):
     """[M, K] float32 (K % 128 == 0) -> (codes uint8 [M, K], scales float32 [M, K/128]).
 
     amax over each 1x128 block, clamped below at 1e-4; data = e4m3(x * (448 / amax))
     with the product formed in fp32; scale = amax / 448.  The reference writes the multiplier as
     ``448.0 / x_amax`` with a Python scalar on the left, which torch evaluates as
     ``reciprocal(x_amax) * 448.0`` (two fp32 roundings, not one division); the same is done here.
+    The scale ``x_amax / 448.0`` is a true division when torch runs the helper on the CPU; on a GPU
+    torch divides a tensor by a Python scalar as ``x_amax * fl(1 / 448)`` (one ulp apart for some
+    values), which is what the reference's callers get: ``scale_via_reciprocal=True`` selects that.
     """
     x = np.asarray(x, dtype=np.float32)
     m, k = x.shape
@@ -35,6 +38,8 @@ def quant_act_1x128(x):
     mult = ((np.float32(1.0) / amax).astype(np.float32) * np.float32(448.0)).astype(np.float32)
     scaled = (xv * mult[:, :, None]).astype(np.float32)
     codes = fp8.e4m3fn_encode_rne(scaled).reshape(m, k)
+    if scale_via_reciprocal:
+        return codes, (amax * (np.float32(1.0) / np.float32(448.0))).astype(np.float32)
     return codes, (amax / np.float32(448.0)).astype(np.float32)
 
 

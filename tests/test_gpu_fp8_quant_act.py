@@ -1,0 +1,83 @@
+"""GPU parity of the FP8 1x128 activation quantiser: bytes and scales bit-exact against the CPU oracle
+(the restatement of per_token_cast_to_fp8, test/test_es_grouped_gemm.py:36-44), through the C ABI."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_blockwise as ofp8
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_capi(x):
+    from expert_specialization_moe_amd import _native
+
+    m, k = x.shape
+    xd = x.cuda()
+    q = torch.full((m, k), 0x55, dtype=torch.uint8, device="cuda")
+    sc = torch.full((m, k // 128), -1.0, dtype=torch.float32, device="cuda")
+    rc = _native.lib.esmoe_fp8_quant_act_1x128(
+        ctypes.c_void_p(xd.data_ptr()), 0 if x.dtype == torch.bfloat16 else 1, ctypes.c_void_p(q.data_ptr()),
+        ctypes.c_void_p(sc.data_ptr()), m, k, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, _native.last_error()
+    torch.cuda.synchronize()
+    return q.cpu().numpy(), sc.cpu().numpy()
+
+
+def _inputs(m, k, dtype, seed):
+    gen = torch.Generator().manual_seed(seed)
+    x = (torch.randn((m, k), generator=gen) * torch.exp(2.0 * torch.randn((m, 1), generator=gen))).to(dtype)
+    if m:
+        x[0, :128] = 0                                   # all-zero block: amax clamps to 1e-4
+        x[m // 2, 128:256] = torch.tensor(3e-5).to(dtype)   # below the clamp
+        x[m - 1, :128] = torch.tensor(448.0).to(dtype)
+        x[m - 1, 5] = torch.tensor(-1.75).to(dtype)
+    return x
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 128), (7, 384), (333, 512), (1030, 7168)])
+def test_quant_act_bit_exact(esmoe, dtype, shape):
+    x = _inputs(*shape, dtype, seed=shape[0])
+    q, sc = _run_capi(x)
+    q_ref, sc_ref = ofp8.quant_act_1x128(H.hp_to_f32(x), scale_via_reciprocal=True)
+    assert np.array_equal(q, q_ref), f"{(q != q_ref).sum()} bytes differ"
+    assert np.array_equal(sc.view(np.uint32), sc_ref.view(np.uint32)), "scales differ"
+
+
+def test_quant_act_matches_torch_helper_and_feeds_the_gemm(esmoe):
+    """Operator path: same bytes as the torch quantiser, and its outputs drive the grouped GEMM."""
+    from expert_specialization_moe_amd import quant as Q
+    from expert_specialization_moe_amd import workloads as W
+
+    prob = W.Problem("ragged", 256, 512, [3, 40, 0, 130])
+    ops = W.make_fp8_blockwise_operands(prob, "cuda", seed=3)
+    gen = torch.Generator().manual_seed(9)
+    x = torch.randn((prob.total_rows, prob.k), generator=gen).to(torch.bfloat16).cuda()
+    q, sc = esmoe.es_fp8_quant_act_1x128(x)
+    q_t, sc_t = Q.quant_act_1x128(x)
+    assert torch.equal(q.view(torch.uint8), q_t.view(torch.uint8)) and torch.equal(sc, sc_t)
+    out = torch.empty_like(ops["output"])
+    esmoe.es_fp8_blockwise_scaled_grouped_mm(out, q, ops["b"], sc, ops["scales_b"], ops["stride_a"], ops["stride_b"],
+                                             ops["stride_d"], ops["problem_sizes"], ops["expert_offsets"], ops["workspace"])
+    torch.cuda.synchronize()
+    ref = ofp8.grouped_mm(q.view(torch.uint8).cpu().numpy(), ops["b_phys"].view(torch.uint8).cpu().numpy(),
+                          sc.cpu().numpy(), ops["scales_b_phys"].cpu().numpy(), [[m, prob.n, prob.k] for m in prob.rows],
+                          W.offsets_of(prob.rows))
+    H.check_grouped(H.f32(out), ref, prob.rows, W.offsets_of(prob.rows), "gemm on device-quantised rows")
+
+
+def test_quant_act_empty_and_rejects(esmoe):
+    from expert_specialization_moe_amd import _native
+
+    x = torch.empty((0, 256), dtype=torch.bfloat16)
+    q, sc = _run_capi(x)
+    assert q.shape == (0, 256) and sc.shape == (0, 2)
+    p = ctypes.c_void_p(16)
+    assert _native.lib.esmoe_fp8_quant_act_1x128(p, 0, p, p, 4, 100, None) == -1
+    assert _native.lib.esmoe_fp8_quant_act_1x128(p, 5, p, p, 4, 128, None) == -1
+    with pytest.raises(RuntimeError, match="align to 128"):
+        esmoe.es_fp8_quant_act_1x128(torch.zeros((2, 100), dtype=torch.bfloat16, device="cuda"))

@@ -150,3 +150,19 @@ def test_calc_diff_properties():
     x = np.arange(12.0).reshape(3, 4)
     assert o.calc_diff(x, x) == pytest.approx(0.0, abs=1e-15)
     assert o.calc_diff(x, -x) == pytest.approx(2.0)
+
+
+def test_quant_act_scale_variants_agree_within_one_ulp():
+    """The GPU flavour of the scale (amax * fl(1/448)) is the CPU flavour (amax / 448) up to one ulp, and
+    the quantised bytes do not depend on the flavour."""
+    import numpy as np
+    from oracle import fp8_blockwise as ofp8
+
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((64, 512)) * np.exp(rng.standard_normal((64, 1)) * 3)).astype(np.float32)
+    q0, s0 = ofp8.quant_act_1x128(x)
+    q1, s1 = ofp8.quant_act_1x128(x, scale_via_reciprocal=True)
+    assert np.array_equal(q0, q1)
+    d = np.abs(s0.view(np.int32).astype(np.int64) - s1.view(np.int32).astype(np.int64))
+    assert d.max() <= 1 and (d == 1).any()
+    assert np.array_equal(s1, s0 if False else (np.maximum(np.abs(x.reshape(64, 4, 128)).max(axis=2), np.float32(1e-4)) * (np.float32(1) / np.float32(448))).astype(np.float32))
