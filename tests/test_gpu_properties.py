@@ -155,3 +155,47 @@ def test_small_k_and_many_experts(esmoe):
         ref = o.grouped_mm(H.codes(ops["a"]), H.codes(ops["b_phys"]), H.f32(ops["scales_a"]), H.f32(ops["scales_b_phys"]),
                            [[m, 256, k] for m in rows], W.offsets_of(rows))
         H.check_grouped(y, ref, rows, W.offsets_of(rows), f"k={k}")
+
+
+@pytest.mark.parametrize("kind", ["fp8_blockwise", "mxfp8"])
+def test_graph_capture_replays_match_eager(esmoe, kind):
+    """The operators enqueue kernels only (no memset nodes, no host reads), so a HIP graph of them can be
+    replayed: every replay, with eager work and synchronisations in between, must reproduce the eager result."""
+    from expert_specialization_moe_amd import workloads as W
+
+    prob = W.Problem("graph", 384, 512, [33, 0, 200, 7, 129], kind=kind)
+    make = W.make_mxfp8_operands if kind == "mxfp8" else W.make_fp8_blockwise_operands
+    ops = make(prob, "cuda", seed=21)
+    # a workspace large enough that the FP8 operator allocates nothing while the graph is recorded
+    ops["workspace"] = torch.zeros((4096,), dtype=torch.uint8, device="cuda")
+
+    def call(out):
+        if kind == "mxfp8":
+            esmoe.es_sm100_mxfp8_blockscaled_grouped_mm(out, ops["a"], ops["b"], ops["sfa"], ops["sfb"], ops["problem_sizes"],
+                                                        ops["expert_offsets"], ops["blockscale_offsets"])
+        else:
+            esmoe.es_fp8_blockwise_scaled_grouped_mm(out, ops["a"], ops["b"], ops["scales_a"], ops["scales_b"],
+                                                     ops["stride_a"], ops["stride_b"], ops["stride_d"], ops["problem_sizes"],
+                                                     ops["expert_offsets"], ops["workspace"])
+
+    eager = torch.zeros_like(ops["output"])
+    call(eager)
+    torch.cuda.synchronize()
+    out = torch.zeros_like(ops["output"])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(out)                      # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(out)
+    for rep in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        scratch = torch.randn(1024, device="cuda").sum().item()   # eager work between replays
+        assert np.isfinite(scratch)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager result"
