@@ -42,9 +42,10 @@ def parse():
     ap.add_argument("--tokens", type=int, default=8192, help="c3 only")
     ap.add_argument("--routing", default="zipf", choices=["zipf", "uniform"], help="c3 only")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--op", default="gemm", choices=["gemm", "quant", "quant_act"],
+    ap.add_argument("--op", default="gemm", choices=["gemm", "quant", "quant_act", "quant_weight"],
                     help="quant: the MXFP8 grouped quantisation of the workload's activation rows (c4 stage 1); "
-                         "quant_act: the FP8 1x128 activation quantisation of the same rows")
+                         "quant_act: the FP8 1x128 activation quantisation of the same rows; "
+                         "quant_weight: the FP8 128x128 quantisation of the workload's [E, N, K] weights")
     ap.add_argument("--force-bm", type=int, default=0, help="single M-tile shape for every expert (0 = device schedule)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -176,6 +177,62 @@ def bench_quant(args, prob, es, W):
     print(json.dumps(out), flush=True)
 
 
+def bench_quant_weight(args, prob, es, W):
+    """FP8 128x128 quantisation of the workload's bf16 weights [E, N, K] (offline operand preparation)."""
+    dev = "cuda:0"
+    e, n, k = prob.num_experts, prob.n, prob.k
+    gen = torch.Generator().manual_seed(args.seed)
+    w1 = (torch.randn((n, k), generator=gen) * 0.02).to(torch.bfloat16)
+    w = w1.to(dev).unsqueeze(0).repeat(e, 1, 1).contiguous()     # same values in every expert: timing does not depend on them
+    q = torch.empty((e, n, k), dtype=torch.uint8, device=dev)
+    sc = torch.empty((e, n // 128, k // 128), dtype=torch.float32, device=dev)
+
+    def step():
+        es.es_fp8_quant_weight_128x128(w, q, sc)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    ms_per_step = start.elapsed_time(stop) / args.steps
+    nbytes = float(e) * n * k * 3 + float(e) * (n // 128) * (k // 128) * 4
+    t = ms_per_step * 1e-3
+    roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": W.HBM_BYTES_PER_S / 1e9, "unit": "GB/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((prob.name, args.op))
+    roof["algorithmic_bytes"] = nbytes
+    roof["roofline_us"] = nbytes / W.HBM_BYTES_PER_S * 1e6
+    out = {
+        "metric": "FP8 128x128 weight quantisation, algorithmic GB/s (bf16 in, e4m3 + fp32 scales out)",
+        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 -> fp8_e4m3 + fp32 scales", "data": "synthetic",
+        "config": {"workload": f"{prob.name} quant_weight: E={e} N={n} K={k} seed={args.seed}"},
+        "roofline": roof,
+    }
+    if args.calibration_copy:
+        calibration_copy()
+    if not args.no_cpu_baseline:
+        from oracle import fp8_blockwise as ofp8
+
+        ws = w1[: min(n, 512)].float().numpy()
+        used, nrows = 0.0, 0
+        while used < args.cpu_seconds:
+            t0 = time.perf_counter()
+            ofp8.quant_weight_128x128(ws)
+            used += time.perf_counter() - t0
+            nrows += ws.shape[0]
+        out["cpu_baseline"] = {"value": nrows * k * 3.0 / used / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"{nrows} weight rows through the numpy oracle ({used:.1f} s)"}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -191,6 +248,9 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
     prob = W.config_problem(args.config, seed=args.seed, tokens=args.tokens, routing=args.routing)
+    if args.op == "quant_weight":
+        bench_quant_weight(args, prob, es, W)
+        return
     if args.op != "gemm":
         bench_quant(args, prob, es, W)
         return

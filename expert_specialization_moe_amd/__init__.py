@@ -13,6 +13,7 @@ from .ops import (  # noqa: F401
     es_sm100_mxfp8_blockscaled_grouped_mm,
     es_sm100_mxfp8_blockscaled_grouped_quant,
     es_fp8_quant_act_1x128,
+    es_fp8_quant_weight_128x128,
 )
 
 __all__ = [
@@ -20,4 +21,5 @@ __all__ = [
     "es_sm100_mxfp8_blockscaled_grouped_mm",
     "es_sm100_mxfp8_blockscaled_grouped_quant",
     "es_fp8_quant_act_1x128",
+    "es_fp8_quant_weight_128x128",
 ]

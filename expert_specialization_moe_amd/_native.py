@@ -42,6 +42,8 @@ lib.esmoe_mxfp8_grouped_quant.restype = _i
 lib.esmoe_mxfp8_grouped_quant.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
 lib.esmoe_fp8_quant_act_1x128.restype = _i
 lib.esmoe_fp8_quant_act_1x128.argtypes = [_vp, _i, _vp, _vp, ctypes.c_long, _i, _vp]
+lib.esmoe_fp8_quant_weight_128x128.restype = _i
+lib.esmoe_fp8_quant_weight_128x128.argtypes = [_vp, _i, _vp, _vp, ctypes.c_long, _i, _vp]
 lib.esmoe_last_error.restype = ctypes.c_char_p
 lib.esmoe_last_error.argtypes = []
 lib.esmoe_version.restype = ctypes.c_char_p

@@ -21,6 +21,9 @@ extern "C" int esmoe_launch_mxfp8_quant(const void* in, int in_dtype, const int*
 extern "C" int esmoe_launch_fp8_quant_act(const void* in, int in_dtype, void* q, float* scales, long total_rows, int k,
                                           hipStream_t stream);
 
+extern "C" int esmoe_launch_fp8_quant_weight(const void* in, int in_dtype, void* q, float* scales, long rows, int k,
+                                             hipStream_t stream);
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -202,6 +205,25 @@ int esmoe_fp8_quant_act_1x128(const void* in, int in_dtype, void* q, float* scal
   int rc = current_device_info(&info);
   if (rc) return rc;
   rc = esmoe_launch_fp8_quant_act(in, in_dtype, q, scales, total_rows, k, (hipStream_t)stream);
+  if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return 0;
+}
+
+int esmoe_fp8_quant_weight_128x128(const void* in, int in_dtype, void* q, float* scales, long rows, int k, void* stream) {
+  g_err[0] = 0;
+  if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must align to 128, got %d", k);
+  if (rows < 0 || rows % 128 || rows / 128 > 65535)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "rows must be a multiple of 128 in [0, 128 * 65535], got %ld", rows);
+  if (in_dtype != ESMOE_IN_BF16 && in_dtype != ESMOE_IN_FP16)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in_dtype must be ESMOE_IN_BF16 or ESMOE_IN_FP16");
+  if (rows == 0) return 0;
+  if (!in || !q || !scales) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if ((uintptr_t)in % 16 || (uintptr_t)q % 8 || (uintptr_t)scales % 4)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in must be 16-byte aligned, q 8-byte aligned, scales 4-byte aligned");
+  DeviceInfo info;
+  int rc = current_device_info(&info);
+  if (rc) return rc;
+  rc = esmoe_launch_fp8_quant_weight(in, in_dtype, q, scales, rows, k, (hipStream_t)stream);
   if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
   return 0;
 }

@@ -1,4 +1,6 @@
-// FP8 1x128 activation quantisation for gfx950: bf16/fp16 rows -> e4m3fn bytes + one fp32 scale
+// FP8 operand quantisers for gfx950 (activations 1x128, weights 128x128).
+//
+// Activations: bf16/fp16 rows -> e4m3fn bytes + one fp32 scale
 // per 128-wide block of a row (the operand format of the FP8-blockwise grouped GEMM).
 //
 // Arithmetic follows the torch helper the reference's callers use, per_token_cast_to_fp8
@@ -74,7 +76,85 @@ fp8_quant_act_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q, f
   }
 }
 
+// 128x128 weight quantisation: the torch helper per_block_cast_to_fp8 (test/test_es_grouped_gemm.py:47-59)
+// applied to the physical [rows, K] matrix (rows = E * N), which equals the reference's route through
+// the transposed (K, N) view (:127,132-134).  One workgroup per 128x128 block: 16 lanes per row
+// segment, 8 passes of 16 rows; the block maximum goes through lane swaps and 4 words of LDS.
+template <bool FP16>
+__global__ void __launch_bounds__(kActQuantThreads) __attribute__((amdgpu_waves_per_eu(4, 8)))
+fp8_quant_weight_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q, float* __restrict__ scales, int k) {
+  __shared__ float s_max[4];
+  const int kt = blockIdx.x, rb = blockIdx.y, tid = threadIdx.x;
+  const int sub = tid & 15, rrow = tid >> 4;
+  const long base = ((long)rb * 128 + rrow) * k + kt * 128 + sub * 8;
+  v4i raw[8];
+#pragma unroll
+  for (int p = 0; p < 8; p++) raw[p] = __builtin_nontemporal_load((const v4i*)(in + base + (long)p * 16 * k));
+  float amax = 0.f;
+#pragma unroll
+  for (int p = 0; p < 8; p++) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t w = (uint32_t)raw[p][i];
+      float a, b;
+      if constexpr (FP16) {
+        a = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+        b = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+      } else {
+        a = __builtin_bit_cast(float, w << 16);
+        b = __builtin_bit_cast(float, w & 0xffff0000u);
+      }
+      amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(a), __builtin_fabsf(b)));
+    }
+  }
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, d));
+  if ((tid & 63) == 0) s_max[tid >> 6] = amax;
+  __syncthreads();
+  amax = __builtin_fmaxf(__builtin_fmaxf(s_max[0], s_max[1]), __builtin_fmaxf(s_max[2], s_max[3]));
+  amax = __builtin_fmaxf(amax, 1e-4f);
+  const float mult = (1.0f / amax) * 448.0f;
+#pragma unroll
+  for (int p = 0; p < 8; p++) {
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t w = (uint32_t)raw[p][i];
+      if constexpr (FP16) {
+        x[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+        x[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+      } else {
+        x[2 * i] = __builtin_bit_cast(float, w << 16);
+        x[2 * i + 1] = __builtin_bit_cast(float, w & 0xffff0000u);
+      }
+    }
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) y[i] = __builtin_amdgcn_fmed3f(x[i] * mult, -448.f, 448.f);
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], 0, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+    __builtin_nontemporal_store(v2i{w0, w1}, (v2i*)(q + base + (long)p * 16 * k));
+  }
+  if (tid == 0) scales[(long)rb * (k >> 7) + kt] = amax * (1.0f / 448.0f);
+}
+
 }  // namespace esmoe
+
+extern "C" int esmoe_launch_fp8_quant_weight(const void* in, int in_dtype, void* q, float* scales, long rows, int k,
+                                             hipStream_t stream) {
+  using namespace esmoe;
+  if (rows == 0) return 0;
+  dim3 grid(k / 128, (unsigned)(rows / 128));
+  if (in_dtype == 1)
+    hipLaunchKernelGGL(fp8_quant_weight_kernel<true>, grid, dim3(kActQuantThreads), 0, stream, (const uint16_t*)in,
+                       (uint8_t*)q, scales, k);
+  else
+    hipLaunchKernelGGL(fp8_quant_weight_kernel<false>, grid, dim3(kActQuantThreads), 0, stream, (const uint16_t*)in,
+                       (uint8_t*)q, scales, k);
+  return (int)hipGetLastError();
+}
 
 extern "C" int esmoe_launch_fp8_quant_act(const void* in, int in_dtype, void* q, float* scales, long total_rows, int k,
                                           hipStream_t stream) {

@@ -237,6 +237,33 @@ void es_fp8_quant_act_1x128(const torch::Tensor& input, torch::Tensor& quant_out
   check_rc(rc, "es_fp8_quant_act_1x128");
 }
 
+// Weight-side companion of es_fp8_quant_act_1x128: per_block_cast_to_fp8
+// (test/test_es_grouped_gemm.py:47-59) on the physical [..., N, K] weight tensor.
+void es_fp8_quant_weight_128x128(const torch::Tensor& input, torch::Tensor& quant_output, torch::Tensor& scales) {
+  TORCH_CHECK(input.dim() >= 2, "input must have at least 2 dimensions");
+  const int64_t k = input.size(-1), n = input.size(-2);
+  TORCH_CHECK(k % 128 == 0 && n % 128 == 0, "n and k must align to 128");
+  TORCH_CHECK(input.scalar_type() == torch::kBFloat16 || input.scalar_type() == torch::kHalf,
+              "dtype must be kFloat16 or kBFloat16");
+  TORCH_CHECK(input.is_contiguous(), "input must be contiguous");
+  const int64_t rows = input.numel() / k;
+  TORCH_CHECK(quant_output.is_contiguous() && quant_output.element_size() == 1 && quant_output.numel() == rows * k,
+              "quant_output must be a contiguous 1-byte tensor with the input's number of elements");
+  TORCH_CHECK(scales.is_contiguous() && scales.scalar_type() == torch::kFloat32 &&
+                  scales.numel() == (rows / 128) * (k / 128),
+              "scales must be a contiguous float32 tensor with one element per 128x128 block");
+  require_device(input, "es_fp8_quant_weight_128x128");
+  TORCH_CHECK(quant_output.device() == input.device() && scales.device() == input.device(),
+              "all tensors must be on the same device");
+  if (rows == 0) return;
+  c10::DeviceGuard guard(input.device());
+  int rc = esmoe_fp8_quant_weight_128x128(input.data_ptr(),
+                                          input.scalar_type() == torch::kBFloat16 ? ESMOE_IN_BF16 : ESMOE_IN_FP16,
+                                          quant_output.data_ptr(), scales.data_ptr<float>(), (long)rows, (int)k,
+                                          current_stream(input));
+  check_rc(rc, "es_fp8_quant_weight_128x128");
+}
+
 TORCH_LIBRARY(expert_specialization, m) {
   m.def(
       "es_fp8_blockwise_scaled_grouped_mm(Tensor output, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, Tensor "
@@ -249,6 +276,7 @@ TORCH_LIBRARY(expert_specialization, m) {
       "es_sm100_mxfp8_blockscaled_grouped_quant(Tensor input, Tensor problem_sizes, Tensor expert_offsets, Tensor "
       "blockscale_offsets, Tensor quant_output, Tensor scale_factor) -> () ");
   m.def("es_fp8_quant_act_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
+  m.def("es_fp8_quant_weight_128x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
@@ -256,6 +284,7 @@ TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
   m.impl("es_sm100_mxfp8_blockscaled_grouped_mm", &es_sm100_mxfp8_blockscaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
+  m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
 }
 
 // Same functions on the CPU key: the checks run, then require_device() raises.
@@ -264,4 +293,5 @@ TORCH_LIBRARY_IMPL(expert_specialization, CPU, m) {
   m.impl("es_sm100_mxfp8_blockscaled_grouped_mm", &es_sm100_mxfp8_blockscaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
+  m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
 }

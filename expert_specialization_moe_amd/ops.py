@@ -42,3 +42,18 @@ def es_fp8_quant_act_1x128(input, quant_output=None, scales=None):
         scales = torch.empty((m, k // 128), dtype=torch.float32, device=input.device)
     _ns.es_fp8_quant_act_1x128.default(input, quant_output, scales)
     return quant_output, scales
+
+
+def es_fp8_quant_weight_128x128(input, quant_output=None, scales=None):
+    """bf16/fp16 [..., N, K] -> (e4m3fn [..., N, K], fp32 scales [..., N/128, K/128]) on the device.
+
+    The weight-side torch helper of the reference's callers (per_block_cast_to_fp8,
+    test/test_es_grouped_gemm.py:47-59) on the physical weight layout, bit for bit.
+    """
+    lead, n, k = input.shape[:-2], input.shape[-2], input.shape[-1]
+    if quant_output is None:
+        quant_output = torch.empty(input.shape, dtype=torch.float8_e4m3fn, device=input.device)
+    if scales is None:
+        scales = torch.empty((*lead, n // 128, k // 128), dtype=torch.float32, device=input.device)
+    _ns.es_fp8_quant_weight_128x128.default(input, quant_output, scales)
+    return quant_output, scales

@@ -114,6 +114,17 @@ int esmoe_fp8_quant_act_1x128(const void* in, int in_dtype, void* q, float* scal
                               void* stream);
 
 /*
+ * FP8 128x128 weight quantisation: bf16/fp16 [rows, K] (rows = E * N, the physical [E, N, K] weight
+ * tensor) -> e4m3fn bytes + one fp32 scale per 128x128 block, the `b` / `scales_b` operands of
+ * esmoe_fp8_blockwise_grouped_mm in their physical layouts ([E, N, K] and [E, N/128, K/128]).
+ * Like the activation quantiser it replaces a torch helper of the reference's callers,
+ * per_block_cast_to_fp8 (test/test_es_grouped_gemm.py:47-59, applied through the transposed view at
+ * :127,132-134,160,166-168), bit for bit.  rows % 128 == 0, K % 128 == 0, rows <= 128 * 65535.
+ */
+int esmoe_fp8_quant_weight_128x128(const void* in, int in_dtype, void* q, float* scales, long rows, int k,
+                                   void* stream);
+
+/*
  * Host mirrors of the device-side tile schedule, for inspection and CPU tests; they touch no GPU.
  * No counterpart in the reference (its schedule lives inside CUTLASS's grouped tile scheduler).
  * esmoe_host_schedule fills `ws_host` (esmoe_gemm_workspace_bytes(E) bytes of host memory) from host

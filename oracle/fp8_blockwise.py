@@ -43,7 +43,7 @@ def quant_act_1x128(x, scale_via_reciprocal=False):
     return codes, (amax / np.float32(448.0)).astype(np.float32)
 
 
-def quant_weight_128x128(w):
+def quant_weight_128x128(w, scale_via_reciprocal=False):
     """[N, K] float32 (both % 128 == 0) -> (codes uint8 [N, K], scales float32 [N/128, K/128]).
 
     The reference quantises the (K, N) view and transposes data and scales back
@@ -58,6 +58,8 @@ def quant_weight_128x128(w):
     mult = ((np.float32(1.0) / amax).astype(np.float32) * np.float32(448.0)).astype(np.float32)
     scaled = (wv * mult[:, None, :, None]).astype(np.float32)
     codes = fp8.e4m3fn_encode_rne(scaled).reshape(n, k)
+    if scale_via_reciprocal:   # torch's GPU evaluation of amax / 448.0, see quant_act_1x128
+        return codes, (amax * (np.float32(1.0) / np.float32(448.0))).astype(np.float32)
     return codes, (amax / np.float32(448.0)).astype(np.float32)
 
 

@@ -81,3 +81,34 @@ def test_quant_act_empty_and_rejects(esmoe):
     assert _native.lib.esmoe_fp8_quant_act_1x128(p, 5, p, p, 4, 128, None) == -1
     with pytest.raises(RuntimeError, match="align to 128"):
         esmoe.es_fp8_quant_act_1x128(torch.zeros((2, 100), dtype=torch.bfloat16, device="cuda"))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 128, 128), (3, 256, 384), (2, 512, 7168)])
+def test_quant_weight_bit_exact(esmoe, dtype, shape):
+    """128x128 weight quantiser through the C ABI: bytes and scales bit-exact against the oracle's restatement
+    of per_block_cast_to_fp8 (test/test_es_grouped_gemm.py:47-59) and against the torch helper on the GPU."""
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import quant as Q
+
+    e, n, k = shape
+    gen = torch.Generator().manual_seed(e * 7 + n)
+    w = (torch.randn((e, n, k), generator=gen) * 0.02 * torch.exp(torch.randn((e, 1, 1), generator=gen))).to(dtype)
+    w[0, :128, :128] = 0                         # all-zero block: amax clamps to 1e-4
+    wd = w.cuda()
+    q = torch.full((e, n, k), 0x55, dtype=torch.uint8, device="cuda")
+    sc = torch.full((e, n // 128, k // 128), -1.0, dtype=torch.float32, device="cuda")
+    rc = _native.lib.esmoe_fp8_quant_weight_128x128(
+        ctypes.c_void_p(wd.data_ptr()), 0 if dtype == torch.bfloat16 else 1, ctypes.c_void_p(q.data_ptr()),
+        ctypes.c_void_p(sc.data_ptr()), e * n, k, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, _native.last_error()
+    torch.cuda.synchronize()
+    for i in range(e):
+        q_ref, sc_ref = ofp8.quant_weight_128x128(H.hp_to_f32(w[i]), scale_via_reciprocal=True)
+        assert np.array_equal(q[i].cpu().numpy(), q_ref), f"expert {i}: bytes differ"
+        assert np.array_equal(sc[i].cpu().numpy().view(np.uint32), sc_ref.view(np.uint32)), f"expert {i}: scales differ"
+    q_t, sc_t = Q.quant_weight_128x128(wd)
+    q_o, sc_o = esmoe.es_fp8_quant_weight_128x128(wd)
+    assert torch.equal(q_o.view(torch.uint8), q_t.view(torch.uint8)) and torch.equal(sc_o, sc_t)
+    assert torch.equal(q_o.view(torch.uint8), q)
+    assert _native.lib.esmoe_fp8_quant_weight_128x128(ctypes.c_void_p(16), 0, ctypes.c_void_p(16), ctypes.c_void_p(16), 100, 128, None) == -1
