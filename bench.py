@@ -42,10 +42,11 @@ def parse():
     ap.add_argument("--tokens", type=int, default=8192, help="c3 only")
     ap.add_argument("--routing", default="zipf", choices=["zipf", "uniform"], help="c3 only")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--op", default="gemm", choices=["gemm", "quant", "quant_act", "quant_weight"],
+    ap.add_argument("--op", default="gemm", choices=["gemm", "quant", "quant_act", "quant_weight", "route"],
                     help="quant: the MXFP8 grouped quantisation of the workload's activation rows (c4 stage 1); "
                          "quant_act: the FP8 1x128 activation quantisation of the same rows; "
-                         "quant_weight: the FP8 128x128 quantisation of the workload's [E, N, K] weights")
+                         "quant_weight: the FP8 128x128 quantisation of the workload's [E, N, K] weights; "
+                         "route: top-k ids -> per-expert metadata + row packing of the workload's routing")
     ap.add_argument("--force-bm", type=int, default=0, help="single M-tile shape for every expert (0 = device schedule)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -177,6 +178,66 @@ def bench_quant(args, prob, es, W):
     print(json.dumps(out), flush=True)
 
 
+def bench_route(args, prob, es, W):
+    """Routing metadata (counts, offsets, packing order) + row packing for the workload's expert row counts:
+    one pair per packed row, in a shuffled order, as a router would emit them."""
+    import numpy as np
+
+    dev = "cuda:0"
+    e, n, k, total = prob.num_experts, prob.n, prob.k, prob.total_rows
+    rng = np.random.default_rng(args.seed)
+    ids = np.repeat(np.arange(e, dtype=np.int32), prob.rows)
+    rng.shuffle(ids)
+    d_ids = torch.from_numpy(ids).to(dev)
+    x = torch.randn((total, k), generator=torch.Generator().manual_seed(args.seed)).to(torch.bfloat16).to(dev)
+    packed = torch.empty_like(x)
+
+    def step():
+        ps, eo, bso, dst = es.es_route_metadata(d_ids, 0, e, n, k)
+        es.es_permute_rows(x, dst, 1, packed)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    ms_per_step = start.elapsed_time(stop) / args.steps
+    nbytes = float(total) * (k * 2 * 2 + 4 * 3)    # rows read and written once, ids read twice, dst_row written
+    t = ms_per_step * 1e-3
+    roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": W.HBM_BYTES_PER_S / 1e9, "unit": "GB/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["algorithmic_bytes"] = nbytes
+    roof["roofline_us"] = nbytes / W.HBM_BYTES_PER_S * 1e6
+    out = {
+        "metric": "routing metadata + row packing, algorithmic GB/s (4 kernels)",
+        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int32 ids, bf16 rows", "data": "synthetic",
+        "config": {"workload": f"{prob.name} route: E={e} K={k} pairs={total} seed={args.seed}"},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        from oracle import routing as oroute
+
+        used, reps = 0.0, 0
+        xs = x[: min(total, 2048)].float().cpu().numpy()
+        while used < args.cpu_seconds:
+            t0 = time.perf_counter()
+            r = oroute.route_metadata(ids, 0, e, n, k)
+            oroute.permute_rows(xs, r[3][: xs.shape[0]] % xs.shape[0], 1, xs.shape[0])
+            used += time.perf_counter() - t0
+            reps += 1
+        out["cpu_baseline"] = {"value": reps * (total * 12.0 + xs.size * 8.0) / used / 1e9, "unit": "GB/s", "cores": 1,
+                               "kind": "port", "sample": f"{reps} passes: all ids, first {xs.shape[0]} rows packed ({used:.1f} s)"}
+    print(json.dumps(out), flush=True)
+
+
 def bench_quant_weight(args, prob, es, W):
     """FP8 128x128 quantisation of the workload's bf16 weights [E, N, K] (offline operand preparation)."""
     dev = "cuda:0"
@@ -250,6 +311,9 @@ def main():
     prob = W.config_problem(args.config, seed=args.seed, tokens=args.tokens, routing=args.routing)
     if args.op == "quant_weight":
         bench_quant_weight(args, prob, es, W)
+        return
+    if args.op == "route":
+        bench_route(args, prob, es, W)
         return
     if args.op != "gemm":
         bench_quant(args, prob, es, W)

@@ -14,6 +14,8 @@ from .ops import (  # noqa: F401
     es_sm100_mxfp8_blockscaled_grouped_quant,
     es_fp8_quant_act_1x128,
     es_fp8_quant_weight_128x128,
+    es_route_metadata,
+    es_permute_rows,
 )
 
 __all__ = [
@@ -22,4 +24,6 @@ __all__ = [
     "es_sm100_mxfp8_blockscaled_grouped_quant",
     "es_fp8_quant_act_1x128",
     "es_fp8_quant_weight_128x128",
+    "es_route_metadata",
+    "es_permute_rows",
 ]

@@ -24,7 +24,7 @@ OBJ = os.path.join(PKG, "build")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
-HIP_SOURCES = ["grouped_gemm.hip", "mxfp8_quant.hip", "fp8_quant.hip", "capi.hip"]
+HIP_SOURCES = ["grouped_gemm.hip", "mxfp8_quant.hip", "fp8_quant.hip", "routing.hip", "capi.hip"]
 HIP_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-mcode-object-version=5",
     # packed fp32 VALU ops are kept out of the device code

@@ -24,7 +24,15 @@ extern "C" int esmoe_launch_fp8_quant_act(const void* in, int in_dtype, void* q,
 extern "C" int esmoe_launch_fp8_quant_weight(const void* in, int in_dtype, void* q, float* scales, long rows, int k,
                                              hipStream_t stream);
 
+extern "C" int esmoe_launch_route_metadata(const int* ids, long num_pairs, int first_expert, int num_experts, int n, int k,
+                                           int* problem_sizes, int* expert_offsets, int* blockscale_offsets, int* dst_row,
+                                           int* chunk_counts, hipStream_t stream);
+extern "C" int esmoe_launch_permute_rows(const void* in, const int* dst_row, long num_pairs, int topk, long row_bytes,
+                                         void* out, hipStream_t stream);
+
 namespace {
+
+constexpr long kRouteChunk = 1024;   // pairs per wavefront in routing.hip
 
 thread_local char g_err[512] = "";
 
@@ -225,6 +233,52 @@ int esmoe_fp8_quant_weight_128x128(const void* in, int in_dtype, void* q, float*
   if (rc) return rc;
   rc = esmoe_launch_fp8_quant_weight(in, in_dtype, q, scales, rows, k, (hipStream_t)stream);
   if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return 0;
+}
+
+size_t esmoe_route_workspace_bytes(long num_pairs, int num_experts) {
+  if (num_pairs < 0) num_pairs = 0;
+  if (num_experts < 1) num_experts = 1;
+  const size_t chunks = (size_t)((num_pairs + kRouteChunk - 1) / kRouteChunk);
+  const size_t bytes = (chunks ? chunks : 1) * (size_t)num_experts * 4;
+  return (bytes + 255) & ~(size_t)255;
+}
+
+int esmoe_route_metadata(const int32_t* topk_ids, long num_pairs, int first_expert, int num_experts, int n, int k,
+                         int32_t* problem_sizes, int32_t* expert_offsets, int32_t* blockscale_offsets,
+                         int32_t* dst_row, void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  if (num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "num_experts must be in [1, %d], got %d", ESMOE_MAX_EXPERTS, num_experts);
+  if (num_pairs < 0 || num_pairs >= (1L << 31))
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "num_pairs must be in [0, 2^31), got %ld", num_pairs);
+  if (!problem_sizes || !expert_offsets || !blockscale_offsets || (num_pairs && (!topk_ids || !dst_row)))
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if (!workspace || workspace_bytes < esmoe_route_workspace_bytes(num_pairs, num_experts))
+    return fail(ESMOE_ERR_WORKSPACE_TOO_SMALL, "workspace needs %zu bytes, got %zu",
+                esmoe_route_workspace_bytes(num_pairs, num_experts), workspace_bytes);
+  DeviceInfo info;
+  int rc = current_device_info(&info);
+  if (rc) return rc;
+  rc = esmoe_launch_route_metadata(topk_ids, num_pairs, first_expert, num_experts, n, k, problem_sizes, expert_offsets,
+                                   blockscale_offsets, dst_row, (int*)workspace, (hipStream_t)stream);
+  if (rc) return fail(rc, "routing launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return 0;
+}
+
+int esmoe_permute_rows(const void* in, const int32_t* dst_row, long num_pairs, int topk, long row_bytes, void* out,
+                       void* stream) {
+  g_err[0] = 0;
+  if (num_pairs < 0 || topk < 1) return fail(ESMOE_ERR_INVALID_ARGUMENT, "num_pairs must be >= 0 and topk >= 1");
+  if (row_bytes <= 0 || row_bytes % 16) return fail(ESMOE_ERR_INVALID_ARGUMENT, "row_bytes must be a positive multiple of 16");
+  if (num_pairs == 0) return 0;
+  if (!in || !dst_row || !out) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if ((uintptr_t)in % 16 || (uintptr_t)out % 16) return fail(ESMOE_ERR_INVALID_ARGUMENT, "in and out must be 16-byte aligned");
+  DeviceInfo info;
+  int rc = current_device_info(&info);
+  if (rc) return rc;
+  rc = esmoe_launch_permute_rows(in, dst_row, num_pairs, topk, row_bytes, out, (hipStream_t)stream);
+  if (rc) return fail(rc, "permute launch failed: %s", hipGetErrorString((hipError_t)rc));
   return 0;
 }
 

@@ -1,0 +1,169 @@
+// Routing metadata on the device: top-k expert ids -> the per-expert tensors the grouped operators
+// consume, plus the row permutation that packs token rows expert by expert.
+//
+// The reference builds these on the host with torch/Python in its tests and benchmark
+// (counts -> expert_offsets prefix sum: benchmark/benchmark_es_fp8_blockwise_moe.py:44-56,72-88;
+// blockscale_offsets = prefix sum of the counts rounded up to 128:
+// test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:42-60).  Here the same integers come out of
+// three small kernels, so a caller never synchronises with the host between routing and the GEMMs.
+//
+//   pair p = (token p / topk, choice p % topk), id = topk_ids[p] - first_expert; local if 0 <= id < E
+//   counts[e]             = number of local pairs with id == e
+//   expert_offsets[e]     = sum of counts[0..e)            (E + 1 entries, the last is the total)
+//   blockscale_offsets[e] = sum of align128(counts[0..e))  (E + 1 entries)
+//   problem_sizes[e]      = (counts[e], n, k)
+//   dst_row[p]            = expert_offsets[id] + (number of local pairs q < p with the same id), or -1
+// The rank is by pair index, so the permutation is stable and the result is deterministic.
+//
+// Pairs are cut into chunks of kChunk; one wavefront owns a chunk.  Pass 1 counts ids per chunk, pass 2
+// (one workgroup, thread = expert) scans the chunk counts of each expert and then the experts, pass 3
+// ranks the pairs of a chunk 64 at a time with running per-expert counters in LDS.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace esmoe {
+
+constexpr int kChunk = 1024;       // pairs per wavefront
+constexpr int kMaxRouteExperts = 1024;
+
+__global__ void __launch_bounds__(64) route_count_kernel(const int* __restrict__ ids, long num_pairs, int first_expert,
+                                                         int num_experts, int* __restrict__ chunk_counts) {
+  __shared__ int s_cnt[kMaxRouteExperts];
+  const int lane = threadIdx.x;
+  for (int e = lane; e < num_experts; e += 64) s_cnt[e] = 0;
+  __syncthreads();
+  const long base = (long)blockIdx.x * kChunk;
+  for (int i = lane; i < kChunk; i += 64) {
+    const long p = base + i;
+    if (p < num_pairs) {
+      const int id = ids[p] - first_expert;
+      if (id >= 0 && id < num_experts) atomicAdd(&s_cnt[id], 1);
+    }
+  }
+  __syncthreads();
+  for (int e = lane; e < num_experts; e += 64) chunk_counts[(long)blockIdx.x * num_experts + e] = s_cnt[e];
+}
+
+__global__ void __launch_bounds__(1024) route_scan_kernel(int* __restrict__ chunk_counts, int num_chunks, int num_experts,
+                                                          int n, int k, int* __restrict__ problem_sizes,
+                                                          int* __restrict__ expert_offsets,
+                                                          int* __restrict__ blockscale_offsets) {
+  __shared__ int s_cnt[kMaxRouteExperts];
+  const int e = threadIdx.x;
+  int total = 0;
+  if (e < num_experts) {
+    // exclusive scan over the chunks, in place: chunk_counts[c][e] becomes the rank base of chunk c
+    for (int c = 0; c < num_chunks; c++) {
+      const long idx = (long)c * num_experts + e;
+      const int v = chunk_counts[idx];
+      chunk_counts[idx] = total;
+      total += v;
+    }
+    s_cnt[e] = total;
+  }
+  __syncthreads();
+  if (e < num_experts) {
+    int off = 0, boff = 0;
+    for (int j = 0; j < e; j++) {
+      const int c = s_cnt[j];
+      off += c;
+      boff += (c + 127) & ~127;
+    }
+    expert_offsets[e] = off;
+    blockscale_offsets[e] = boff;
+    problem_sizes[e * 3 + 0] = total;
+    problem_sizes[e * 3 + 1] = n;
+    problem_sizes[e * 3 + 2] = k;
+    if (e == num_experts - 1) {
+      expert_offsets[num_experts] = off + total;
+      blockscale_offsets[num_experts] = boff + ((total + 127) & ~127);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(64) route_rank_kernel(const int* __restrict__ ids, long num_pairs, int first_expert,
+                                                        int num_experts, const int* __restrict__ chunk_base,
+                                                        const int* __restrict__ expert_offsets,
+                                                        int* __restrict__ dst_row) {
+  __shared__ int s_run[kMaxRouteExperts];   // next free row of every expert for this chunk
+  const int lane = threadIdx.x;
+  for (int e = lane; e < num_experts; e += 64) s_run[e] = expert_offsets[e] + chunk_base[(long)blockIdx.x * num_experts + e];
+  __syncthreads();
+  const long base = (long)blockIdx.x * kChunk;
+  for (int step = 0; step < kChunk / 64; step++) {
+    const long p = base + step * 64 + lane;
+    if (base + step * 64 >= num_pairs) break;   // wave-uniform
+    int id = -1;
+    if (p < num_pairs) {
+      id = ids[p] - first_expert;
+      if (id < 0 || id >= num_experts) id = -1;
+    }
+    int row = -1;
+    // group the lanes by id: every round settles the lanes that share the id of the first unsettled lane
+    unsigned long long todo = __ballot(id >= 0);
+    while (todo) {
+      const int leader = __builtin_ctzll(todo);
+      const int lid = __shfl(id, leader);
+      const unsigned long long same = __ballot(id == lid);
+      if (id == lid) {
+        const int before = __builtin_popcountll(same & ((1ull << lane) - 1ull));
+        row = s_run[lid] + before;
+      }
+      __builtin_amdgcn_wave_barrier();
+      if (lane == leader) s_run[lid] += __builtin_popcountll(same);
+      __builtin_amdgcn_wave_barrier();
+      todo &= ~same;
+    }
+    if (p < num_pairs) dst_row[p] = row;
+  }
+}
+
+// Packs rows for the grouped operators: out[dst_row[p], :] = in[p / topk, :] for every local pair
+// (2-byte elements, row_bytes a multiple of 16).  One wavefront moves one row in 1 KB steps.
+__global__ void __launch_bounds__(256) permute_rows_kernel(const uint8_t* __restrict__ in, const int* __restrict__ dst_row,
+                                                           long num_pairs, int topk, long row_bytes,
+                                                           uint8_t* __restrict__ out) {
+  typedef int v4i __attribute__((ext_vector_type(4)));
+  const long p = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (p >= num_pairs) return;
+  const int dst = dst_row[p];
+  if (dst < 0) return;
+  const uint8_t* src = in + (p / topk) * row_bytes;
+  uint8_t* d = out + (long)dst * row_bytes;
+  for (long off = (threadIdx.x & 63) * 16; off < row_bytes; off += 4096) {
+    v4i v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (off + u * 1024 < row_bytes) v[u] = __builtin_nontemporal_load((const v4i*)(src + off + u * 1024));
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (off + u * 1024 < row_bytes) __builtin_nontemporal_store(v[u], (v4i*)(d + off + u * 1024));
+  }
+}
+
+}  // namespace esmoe
+
+extern "C" int esmoe_launch_route_metadata(const int* ids, long num_pairs, int first_expert, int num_experts, int n, int k,
+                                           int* problem_sizes, int* expert_offsets, int* blockscale_offsets, int* dst_row,
+                                           int* chunk_counts, hipStream_t stream) {
+  using namespace esmoe;
+  const int chunks = (int)((num_pairs + kChunk - 1) / kChunk);
+  if (chunks > 0)
+    hipLaunchKernelGGL(route_count_kernel, dim3(chunks), dim3(64), 0, stream, ids, num_pairs, first_expert, num_experts,
+                       chunk_counts);
+  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3((num_experts + 63) & ~63), 0, stream, chunk_counts, chunks,
+                     num_experts, n, k, problem_sizes, expert_offsets, blockscale_offsets);
+  if (chunks > 0)
+    hipLaunchKernelGGL(route_rank_kernel, dim3(chunks), dim3(64), 0, stream, ids, num_pairs, first_expert, num_experts,
+                       chunk_counts, expert_offsets, dst_row);
+  return (int)hipGetLastError();
+}
+
+extern "C" int esmoe_launch_permute_rows(const void* in, const int* dst_row, long num_pairs, int topk, long row_bytes,
+                                         void* out, hipStream_t stream) {
+  using namespace esmoe;
+  if (num_pairs == 0) return 0;
+  hipLaunchKernelGGL(permute_rows_kernel, dim3((unsigned)((num_pairs + 3) / 4)), dim3(256), 0, stream, (const uint8_t*)in,
+                     dst_row, num_pairs, topk, row_bytes, (uint8_t*)out);
+  return (int)hipGetLastError();
+}

@@ -237,6 +237,49 @@ void es_fp8_quant_act_1x128(const torch::Tensor& input, torch::Tensor& quant_out
   check_rc(rc, "es_fp8_quant_act_1x128");
 }
 
+// Routing metadata and row packing on the device (no counterpart among the reference's operators; its
+// callers build these tensors on the host, benchmark/benchmark_es_fp8_blockwise_moe.py:44-56,72-88).
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> es_route_metadata(const torch::Tensor& topk_ids,
+                                                                                         int64_t first_expert,
+                                                                                         int64_t num_experts, int64_t n,
+                                                                                         int64_t k) {
+  TORCH_CHECK(topk_ids.scalar_type() == torch::kInt32 && topk_ids.is_contiguous(), "topk_ids must be contiguous int32");
+  TORCH_CHECK(num_experts >= 1 && num_experts <= ESMOE_MAX_EXPERTS, "num_experts must be in [1, 1024]");
+  require_device(topk_ids, "es_route_metadata");
+  c10::DeviceGuard guard(topk_ids.device());
+  const int64_t pairs = topk_ids.numel();
+  auto opts = topk_ids.options();
+  torch::Tensor ps = torch::empty({num_experts, 3}, opts), eo = torch::empty({num_experts + 1}, opts),
+                bso = torch::empty({num_experts + 1}, opts), dst = torch::empty({pairs}, opts);
+  torch::Tensor ws = torch::empty({(int64_t)esmoe_route_workspace_bytes((long)pairs, (int)num_experts)},
+                                  opts.dtype(torch::kUInt8));
+  int rc = esmoe_route_metadata(pairs ? topk_ids.data_ptr<int32_t>() : nullptr, (long)pairs, (int)first_expert,
+                                (int)num_experts, (int)n, (int)k, ps.data_ptr<int32_t>(), eo.data_ptr<int32_t>(),
+                                bso.data_ptr<int32_t>(), pairs ? dst.data_ptr<int32_t>() : nullptr, ws.data_ptr(),
+                                ws.nbytes(), current_stream(topk_ids));
+  check_rc(rc, "es_route_metadata");
+  return {ps, eo, bso, dst};
+}
+
+void es_permute_rows(const torch::Tensor& input, const torch::Tensor& dst_row, int64_t topk, torch::Tensor& output) {
+  TORCH_CHECK(input.dim() == 2 && output.dim() == 2 && input.is_contiguous() && output.is_contiguous(),
+              "input and output must be contiguous 2D tensors");
+  TORCH_CHECK(input.size(1) == output.size(1) && input.scalar_type() == output.scalar_type(),
+              "input and output must have the same row length and dtype");
+  TORCH_CHECK(dst_row.scalar_type() == torch::kInt32 && dst_row.is_contiguous(), "dst_row must be contiguous int32");
+  TORCH_CHECK(topk >= 1 && dst_row.numel() == input.size(0) * topk, "dst_row must have rows * topk entries");
+  const int64_t row_bytes = input.size(1) * input.element_size();
+  TORCH_CHECK(row_bytes % 16 == 0, "rows must be a multiple of 16 bytes");
+  require_device(input, "es_permute_rows");
+  TORCH_CHECK(dst_row.device() == input.device() && output.device() == input.device(),
+              "all tensors must be on the same device");
+  if (dst_row.numel() == 0) return;
+  c10::DeviceGuard guard(input.device());
+  int rc = esmoe_permute_rows(input.data_ptr(), dst_row.data_ptr<int32_t>(), (long)dst_row.numel(), (int)topk,
+                              (long)row_bytes, output.data_ptr(), current_stream(input));
+  check_rc(rc, "es_permute_rows");
+}
+
 // Weight-side companion of es_fp8_quant_act_1x128: per_block_cast_to_fp8
 // (test/test_es_grouped_gemm.py:47-59) on the physical [..., N, K] weight tensor.
 void es_fp8_quant_weight_128x128(const torch::Tensor& input, torch::Tensor& quant_output, torch::Tensor& scales) {
@@ -277,6 +320,8 @@ TORCH_LIBRARY(expert_specialization, m) {
       "blockscale_offsets, Tensor quant_output, Tensor scale_factor) -> () ");
   m.def("es_fp8_quant_act_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def("es_fp8_quant_weight_128x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
+  m.def("es_route_metadata(Tensor topk_ids, int first_expert, int num_experts, int n, int k) -> (Tensor, Tensor, Tensor, Tensor)");
+  m.def("es_permute_rows(Tensor input, Tensor dst_row, int topk, Tensor output) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
@@ -285,6 +330,8 @@ TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
+  m.impl("es_route_metadata", &es_route_metadata);
+  m.impl("es_permute_rows", &es_permute_rows);
 }
 
 // Same functions on the CPU key: the checks run, then require_device() raises.
@@ -294,4 +341,6 @@ TORCH_LIBRARY_IMPL(expert_specialization, CPU, m) {
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
+  m.impl("es_route_metadata", &es_route_metadata);
+  m.impl("es_permute_rows", &es_permute_rows);
 }

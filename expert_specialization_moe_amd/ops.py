@@ -57,3 +57,19 @@ def es_fp8_quant_weight_128x128(input, quant_output=None, scales=None):
         scales = torch.empty((*lead, n // 128, k // 128), dtype=torch.float32, device=input.device)
     _ns.es_fp8_quant_weight_128x128.default(input, quant_output, scales)
     return quant_output, scales
+
+
+def es_route_metadata(topk_ids, first_expert, num_experts, n, k):
+    """int32 top-k expert ids [T, topk] -> (problem_sizes [E,3], expert_offsets [E+1], blockscale_offsets [E+1],
+    dst_row [T*topk]) on the device, never touching the host.
+
+    The reference's callers compute these with Python loops on the host
+    (benchmark/benchmark_es_fp8_blockwise_moe.py:44-56,72-88).  Pass ``expert_offsets[:E]`` and
+    ``blockscale_offsets[:E]`` to the grouped operators; the last entries are the packed row totals.
+    """
+    return _ns.es_route_metadata.default(topk_ids.reshape(-1), first_expert, num_experts, n, k)
+
+
+def es_permute_rows(input, dst_row, topk, output):
+    """output[dst_row[p]] = input[p // topk] for every pair with dst_row[p] >= 0 (rows packed by expert)."""
+    _ns.es_permute_rows.default(input, dst_row, topk, output)

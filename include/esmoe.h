@@ -125,6 +125,31 @@ int esmoe_fp8_quant_weight_128x128(const void* in, int in_dtype, void* q, float*
                                    void* stream);
 
 /*
+ * Routing metadata on the device: top-k expert ids -> the per-expert tensors the operators above take.
+ * The reference's callers build these on the host (counts and their prefix sum:
+ * benchmark/benchmark_es_fp8_blockwise_moe.py:44-56,72-88; blockscale_offsets as the prefix sum of the
+ * counts rounded up to 128: test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:42-60); there is no
+ * operator for it in the reference.
+ *
+ *   topk_ids [num_pairs] int32: expert id of pair p = (token p / topk, choice p % topk); ids outside
+ *            [first_expert, first_expert + num_experts) belong to other devices and are skipped
+ *   problem_sizes [E,3] = (count_e, n, k);  expert_offsets [E+1], blockscale_offsets [E+1]: exclusive prefix
+ *            sums of the counts and of the counts rounded up to 128, last entry = total
+ *   dst_row [num_pairs]: row of pair p in the packed [sum count, .] tensors (pairs of one expert keep
+ *            their order, so the result is deterministic), -1 for skipped pairs
+ *   workspace: esmoe_route_workspace_bytes(num_pairs, num_experts) bytes of device scratch
+ */
+size_t esmoe_route_workspace_bytes(long num_pairs, int num_experts);
+int esmoe_route_metadata(const int32_t* topk_ids, long num_pairs, int first_expert, int num_experts, int n, int k,
+                         int32_t* problem_sizes, int32_t* expert_offsets, int32_t* blockscale_offsets,
+                         int32_t* dst_row, void* workspace, size_t workspace_bytes, void* stream);
+
+/* out[dst_row[p], :] = in[p / topk, :] for every pair with dst_row[p] >= 0; rows of row_bytes bytes
+ * (a multiple of 16), `in` and `out` 16-byte aligned.  No counterpart in the reference. */
+int esmoe_permute_rows(const void* in, const int32_t* dst_row, long num_pairs, int topk, long row_bytes, void* out,
+                       void* stream);
+
+/*
  * Host mirrors of the device-side tile schedule, for inspection and CPU tests; they touch no GPU.
  * No counterpart in the reference (its schedule lives inside CUTLASS's grouped tile scheduler).
  * esmoe_host_schedule fills `ws_host` (esmoe_gemm_workspace_bytes(E) bytes of host memory) from host
