@@ -42,11 +42,12 @@ def parse():
     ap.add_argument("--tokens", type=int, default=8192, help="c3 only")
     ap.add_argument("--routing", default="zipf", choices=["zipf", "uniform"], help="c3 only")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--op", default="gemm", choices=["gemm", "quant", "quant_act", "quant_weight", "route"],
+    ap.add_argument("--op", default="gemm", choices=["gemm", "quant", "quant_act", "quant_weight", "route", "swiglu_quant"],
                     help="quant: the MXFP8 grouped quantisation of the workload's activation rows (c4 stage 1); "
                          "quant_act: the FP8 1x128 activation quantisation of the same rows; "
                          "quant_weight: the FP8 128x128 quantisation of the workload's [E, N, K] weights; "
-                         "route: top-k ids -> per-expert metadata + row packing of the workload's routing")
+                         "route: top-k ids -> per-expert metadata + row packing of the workload's routing; "
+                         "swiglu_quant: fused SwiGLU + 1x128 quantisation of the workload's [rows, N] output")
     ap.add_argument("--force-bm", type=int, default=0, help="single M-tile shape for every expert (0 = device schedule)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -171,6 +172,61 @@ def bench_quant(args, prob, es, W):
         while used < args.cpu_seconds:
             t0 = time.perf_counter()
             ofp8.quant_act_1x128(xs) if act else omx.quant_rows(xs)
+            used += time.perf_counter() - t0
+            nrows += xs.shape[0]
+        out["cpu_baseline"] = {"value": nbytes / total * nrows / used / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"{nrows} rows of the same input through the numpy oracle ({used:.1f} s)"}
+    print(json.dumps(out), flush=True)
+
+
+def bench_swiglu_quant(args, prob, es, W):
+    """Fused SwiGLU + FP8 1x128 quantisation of a [rows, N] gate_up output (N = 2 * inter)."""
+    dev = "cuda:0"
+    total, inter = prob.total_rows, prob.n // 2
+    x = torch.randn((total, 2 * inter), generator=torch.Generator().manual_seed(args.seed)).to(torch.bfloat16)
+    xd = x.to(dev)
+    q = torch.empty((total, inter), dtype=torch.uint8, device=dev)
+    sc = torch.empty((total, inter // 128), dtype=torch.float32, device=dev)
+
+    def step():
+        es.es_swiglu_quant_1x128(xd, q, sc)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    ms_per_step = start.elapsed_time(stop) / args.steps
+    nbytes = float(total) * inter * (4 + 1 + 4 / 128.0)
+    t = ms_per_step * 1e-3
+    roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": W.HBM_BYTES_PER_S / 1e9, "unit": "GB/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["algorithmic_bytes"] = nbytes
+    roof["roofline_us"] = nbytes / W.HBM_BYTES_PER_S * 1e6
+    out = {
+        "metric": "fused SwiGLU + FP8 1x128 quantisation, algorithmic GB/s (bf16 [rows, 2I] in, e4m3 + fp32 scales out)",
+        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 -> fp32 -> bf16 -> fp8_e4m3 + fp32 scales", "data": "synthetic",
+        "config": {"workload": f"{prob.name} swiglu_quant: rows={total} inter={inter} seed={args.seed}"},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        import numpy as np
+        from oracle import fp8_blockwise as ofp8
+
+        xs = x[: min(total, 256)].float().numpy()
+        used, nrows = 0.0, 0
+        while used < args.cpu_seconds:
+            t0 = time.perf_counter()
+            with np.errstate(over="ignore"):
+                ofp8.quant_act_1x128(ofp8.swiglu(xs))
             used += time.perf_counter() - t0
             nrows += xs.shape[0]
         out["cpu_baseline"] = {"value": nbytes / total * nrows / used / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
@@ -314,6 +370,9 @@ def main():
         return
     if args.op == "route":
         bench_route(args, prob, es, W)
+        return
+    if args.op == "swiglu_quant":
+        bench_swiglu_quant(args, prob, es, W)
         return
     if args.op != "gemm":
         bench_quant(args, prob, es, W)

@@ -16,6 +16,7 @@ from .ops import (  # noqa: F401
     es_fp8_quant_weight_128x128,
     es_route_metadata,
     es_permute_rows,
+    es_swiglu_quant_1x128,
 )
 
 __all__ = [
@@ -26,4 +27,5 @@ __all__ = [
     "es_fp8_quant_weight_128x128",
     "es_route_metadata",
     "es_permute_rows",
+    "es_swiglu_quant_1x128",
 ]

@@ -50,6 +50,8 @@ lib.esmoe_route_metadata.restype = _i
 lib.esmoe_route_metadata.argtypes = [_vp, ctypes.c_long, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp]
 lib.esmoe_permute_rows.restype = _i
 lib.esmoe_permute_rows.argtypes = [_vp, _vp, ctypes.c_long, _i, ctypes.c_long, _vp, _vp]
+lib.esmoe_swiglu_quant_1x128.restype = _i
+lib.esmoe_swiglu_quant_1x128.argtypes = [_vp, _i, _vp, _vp, ctypes.c_long, _i, _vp]
 lib.esmoe_last_error.restype = ctypes.c_char_p
 lib.esmoe_last_error.argtypes = []
 lib.esmoe_version.restype = ctypes.c_char_p

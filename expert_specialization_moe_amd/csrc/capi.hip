@@ -30,6 +30,9 @@ extern "C" int esmoe_launch_route_metadata(const int* ids, long num_pairs, int f
 extern "C" int esmoe_launch_permute_rows(const void* in, const int* dst_row, long num_pairs, int topk, long row_bytes,
                                          void* out, hipStream_t stream);
 
+extern "C" int esmoe_launch_swiglu_quant(const void* in, int in_dtype, void* q, float* scales, long total_rows, int inter,
+                                        hipStream_t stream);
+
 namespace {
 
 constexpr long kRouteChunk = 1024;   // pairs per wavefront in routing.hip
@@ -233,6 +236,26 @@ int esmoe_fp8_quant_weight_128x128(const void* in, int in_dtype, void* q, float*
   if (rc) return rc;
   rc = esmoe_launch_fp8_quant_weight(in, in_dtype, q, scales, rows, k, (hipStream_t)stream);
   if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return 0;
+}
+
+int esmoe_swiglu_quant_1x128(const void* in, int in_dtype, void* q, float* scales, long total_rows, int inter,
+                             void* stream) {
+  g_err[0] = 0;
+  if (inter <= 0 || inter % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "inter must align to 128, got %d", inter);
+  if (in_dtype != ESMOE_IN_BF16 && in_dtype != ESMOE_IN_FP16)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in_dtype must be ESMOE_IN_BF16 or ESMOE_IN_FP16");
+  if (total_rows < 0 || total_rows > (1L << 40) / inter)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "total_rows out of range: %ld", total_rows);
+  if (total_rows == 0) return 0;
+  if (!in || !q || !scales) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if ((uintptr_t)in % 16 || (uintptr_t)q % 8 || (uintptr_t)scales % 4)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in must be 16-byte aligned, q 8-byte aligned, scales 4-byte aligned");
+  DeviceInfo info;
+  int rc = current_device_info(&info);
+  if (rc) return rc;
+  rc = esmoe_launch_swiglu_quant(in, in_dtype, q, scales, total_rows, inter, (hipStream_t)stream);
+  if (rc) return fail(rc, "swiglu quant launch failed: %s", hipGetErrorString((hipError_t)rc));
   return 0;
 }
 

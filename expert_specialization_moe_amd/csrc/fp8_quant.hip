@@ -76,6 +76,82 @@ fp8_quant_act_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q, f
   }
 }
 
+// Fused SwiGLU + 1x128 quantisation: the glue between the gate_up and the down projection of an
+// expert MLP.  in [M, 2*I]: gate = in[:, :I], up = in[:, I:];  h = cast(silu(gate) * up) with the
+// product formed in fp32 and rounded once to the input type (what a fused silu-and-mul kernel
+// stores), silu(x) = x / (1 + exp(-x)); then h is quantised exactly as fp8_quant_act_kernel does.
+// Saves one write and one read of the [M, I] intermediate.  No counterpart in the reference.
+template <bool FP16>
+__global__ void __launch_bounds__(kActQuantThreads) __attribute__((amdgpu_waves_per_eu(4, 8)))
+swiglu_quant_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q, float* __restrict__ scales, long chunks,
+                    int inter) {
+  const int cpr = inter >> 3;   // 8-element chunks per output row
+  const long first = ((long)blockIdx.x * 2) * kActQuantThreads + threadIdx.x;
+  v4i rg[2], ru[2];
+#pragma unroll
+  for (int u = 0; u < 2; u++) {
+    const long c = first + (long)u * kActQuantThreads;
+    rg[u] = v4i{0, 0, 0, 0};
+    ru[u] = v4i{0, 0, 0, 0};
+    if (c < chunks) {
+      const long row = c / cpr;
+      const long col = (c - row * cpr) * 8;
+      const uint16_t* g = in + row * 2 * inter + col;
+      rg[u] = __builtin_nontemporal_load((const v4i*)g);
+      ru[u] = __builtin_nontemporal_load((const v4i*)(g + inter));
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 2; u++) {
+    const long c = first + (long)u * kActQuantThreads;
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t wg = (uint32_t)rg[u][i], wu = (uint32_t)ru[u][i];
+      float g0, g1, u0, u1;
+      if constexpr (FP16) {
+        g0 = (float)__builtin_bit_cast(_Float16, (uint16_t)(wg & 0xffffu));
+        g1 = (float)__builtin_bit_cast(_Float16, (uint16_t)(wg >> 16));
+        u0 = (float)__builtin_bit_cast(_Float16, (uint16_t)(wu & 0xffffu));
+        u1 = (float)__builtin_bit_cast(_Float16, (uint16_t)(wu >> 16));
+      } else {
+        g0 = __builtin_bit_cast(float, wg << 16);
+        g1 = __builtin_bit_cast(float, wg & 0xffff0000u);
+        u0 = __builtin_bit_cast(float, wu << 16);
+        u1 = __builtin_bit_cast(float, wu & 0xffff0000u);
+      }
+      const float h0 = (g0 / (1.0f + expf(-g0))) * u0, h1 = (g1 / (1.0f + expf(-g1))) * u1;
+      if constexpr (FP16) {
+        x[2 * i] = (float)(_Float16)h0;
+        x[2 * i + 1] = (float)(_Float16)h1;
+      } else {
+        x[2 * i] = (float)(__bf16)h0;
+        x[2 * i + 1] = (float)(__bf16)h1;
+      }
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) amax = __builtin_fmaxf(amax, __builtin_fabsf(x[i]));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 1));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 2));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 4));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 8));
+    amax = __builtin_fmaxf(amax, 1e-4f);
+    const float mult = (1.0f / amax) * 448.0f;
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) y[i] = __builtin_amdgcn_fmed3f(x[i] * mult, -448.f, 448.f);
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], 0, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+    if (c < chunks) {
+      __builtin_nontemporal_store(v2i{w0, w1}, (v2i*)(q + c * 8));
+      if ((threadIdx.x & 15) == 0) scales[c >> 4] = amax * (1.0f / 448.0f);
+    }
+  }
+}
+
 // 128x128 weight quantisation: the torch helper per_block_cast_to_fp8 (test/test_es_grouped_gemm.py:47-59)
 // applied to the physical [rows, K] matrix (rows = E * N), which equals the reference's route through
 // the transposed (K, N) view (:127,132-134).  One workgroup per 128x128 block: 16 lanes per row
@@ -153,6 +229,22 @@ extern "C" int esmoe_launch_fp8_quant_weight(const void* in, int in_dtype, void*
   else
     hipLaunchKernelGGL(fp8_quant_weight_kernel<false>, grid, dim3(kActQuantThreads), 0, stream, (const uint16_t*)in,
                        (uint8_t*)q, scales, k);
+  return (int)hipGetLastError();
+}
+
+extern "C" int esmoe_launch_swiglu_quant(const void* in, int in_dtype, void* q, float* scales, long total_rows, int inter,
+                                        hipStream_t stream) {
+  using namespace esmoe;
+  const long chunks = total_rows * (long)inter / 8;
+  if (chunks == 0) return 0;
+  const long per_wg = (long)kActQuantThreads * 2;
+  const long grid = (chunks + per_wg - 1) / per_wg;
+  if (in_dtype == 1)
+    hipLaunchKernelGGL(swiglu_quant_kernel<true>, dim3((unsigned)grid), dim3(kActQuantThreads), 0, stream,
+                       (const uint16_t*)in, (uint8_t*)q, scales, chunks, inter);
+  else
+    hipLaunchKernelGGL(swiglu_quant_kernel<false>, dim3((unsigned)grid), dim3(kActQuantThreads), 0, stream,
+                       (const uint16_t*)in, (uint8_t*)q, scales, chunks, inter);
   return (int)hipGetLastError();
 }
 

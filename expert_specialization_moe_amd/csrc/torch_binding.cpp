@@ -237,6 +237,28 @@ void es_fp8_quant_act_1x128(const torch::Tensor& input, torch::Tensor& quant_out
   check_rc(rc, "es_fp8_quant_act_1x128");
 }
 
+// Fused SwiGLU + 1x128 quantisation (no counterpart in the reference).
+void es_swiglu_quant_1x128(const torch::Tensor& input, torch::Tensor& quant_output, torch::Tensor& scales) {
+  TORCH_CHECK(input.dim() == 2 && input.is_contiguous(), "input must be a contiguous 2D tensor");
+  TORCH_CHECK(input.size(1) % 256 == 0, "the row length must be 2 * inter with inter aligned to 128");
+  TORCH_CHECK(input.scalar_type() == torch::kBFloat16 || input.scalar_type() == torch::kHalf,
+              "dtype must be kFloat16 or kBFloat16");
+  const int64_t rows = input.size(0), inter = input.size(1) / 2;
+  TORCH_CHECK(quant_output.is_contiguous() && quant_output.element_size() == 1 && quant_output.numel() == rows * inter,
+              "quant_output must be a contiguous 1-byte tensor of rows * inter elements");
+  TORCH_CHECK(scales.is_contiguous() && scales.scalar_type() == torch::kFloat32 && scales.numel() == rows * (inter / 128),
+              "scales must be a contiguous float32 tensor of rows * inter / 128 elements");
+  require_device(input, "es_swiglu_quant_1x128");
+  TORCH_CHECK(quant_output.device() == input.device() && scales.device() == input.device(),
+              "all tensors must be on the same device");
+  if (rows == 0) return;
+  c10::DeviceGuard guard(input.device());
+  int rc = esmoe_swiglu_quant_1x128(input.data_ptr(), input.scalar_type() == torch::kBFloat16 ? ESMOE_IN_BF16 : ESMOE_IN_FP16,
+                                    quant_output.data_ptr(), scales.data_ptr<float>(), (long)rows, (int)inter,
+                                    current_stream(input));
+  check_rc(rc, "es_swiglu_quant_1x128");
+}
+
 // Routing metadata and row packing on the device (no counterpart among the reference's operators; its
 // callers build these tensors on the host, benchmark/benchmark_es_fp8_blockwise_moe.py:44-56,72-88).
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> es_route_metadata(const torch::Tensor& topk_ids,
@@ -320,6 +342,7 @@ TORCH_LIBRARY(expert_specialization, m) {
       "blockscale_offsets, Tensor quant_output, Tensor scale_factor) -> () ");
   m.def("es_fp8_quant_act_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def("es_fp8_quant_weight_128x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
+  m.def("es_swiglu_quant_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def("es_route_metadata(Tensor topk_ids, int first_expert, int num_experts, int n, int k) -> (Tensor, Tensor, Tensor, Tensor)");
   m.def("es_permute_rows(Tensor input, Tensor dst_row, int topk, Tensor output) -> ()");
 }
@@ -330,6 +353,7 @@ TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
+  m.impl("es_swiglu_quant_1x128", &es_swiglu_quant_1x128);
   m.impl("es_route_metadata", &es_route_metadata);
   m.impl("es_permute_rows", &es_permute_rows);
 }
@@ -341,6 +365,7 @@ TORCH_LIBRARY_IMPL(expert_specialization, CPU, m) {
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
+  m.impl("es_swiglu_quant_1x128", &es_swiglu_quant_1x128);
   m.impl("es_route_metadata", &es_route_metadata);
   m.impl("es_permute_rows", &es_permute_rows);
 }

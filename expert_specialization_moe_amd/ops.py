@@ -73,3 +73,16 @@ def es_route_metadata(topk_ids, first_expert, num_experts, n, k):
 def es_permute_rows(input, dst_row, topk, output):
     """output[dst_row[p]] = input[p // topk] for every pair with dst_row[p] >= 0 (rows packed by expert)."""
     _ns.es_permute_rows.default(input, dst_row, topk, output)
+
+
+def es_swiglu_quant_1x128(input, quant_output=None, scales=None):
+    """bf16/fp16 gate_up output [M, 2*I] -> (e4m3fn [M, I], fp32 scales [M, I/128]) of silu(gate) * up:
+    the down projection's ``a`` / ``scales_a`` in one pass (no counterpart in the reference)."""
+    m, two_i = input.shape
+    inter = two_i // 2
+    if quant_output is None:
+        quant_output = torch.empty((m, inter), dtype=torch.float8_e4m3fn, device=input.device)
+    if scales is None:
+        scales = torch.empty((m, inter // 128), dtype=torch.float32, device=input.device)
+    _ns.es_swiglu_quant_1x128.default(input, quant_output, scales)
+    return quant_output, scales

@@ -125,6 +125,20 @@ int esmoe_fp8_quant_weight_128x128(const void* in, int in_dtype, void* q, float*
                                    void* stream);
 
 /*
+ * Fused SwiGLU + 1x128 quantisation between the gate_up and the down projection:
+ *   in [total_rows, 2*inter] bf16/fp16 (gate = first half of a row, up = second half)
+ *   h = cast_to_in_dtype(silu(gate) * up)   (fp32 product, one rounding; silu(x) = x / (1 + exp(-x)))
+ *   q [total_rows, inter], scales [total_rows, inter/128] = the 1x128 quantisation of h, as
+ *   esmoe_fp8_quant_act_1x128 computes it.   inter % 128 == 0.
+ * No counterpart in the reference (its benchmark shapes pair a gate_up N = 2*inter with a down
+ * K = inter, benchmark/benchmark_es_fp8_blockwise_moe.py:349-364, and leave the step between to the caller).
+ * exp() is the device's fp32 routine, so bytes can differ from a host evaluation where a product
+ * falls within an ulp of a rounding boundary; the parity test states the tolerance.
+ */
+int esmoe_swiglu_quant_1x128(const void* in, int in_dtype, void* q, float* scales, long total_rows, int inter,
+                             void* stream);
+
+/*
  * Routing metadata on the device: top-k expert ids -> the per-expert tensors the operators above take.
  * The reference's callers build these on the host (counts and their prefix sum:
  * benchmark/benchmark_es_fp8_blockwise_moe.py:44-56,72-88; blockscale_offsets as the prefix sum of the

@@ -43,6 +43,20 @@ def quant_act_1x128(x, scale_via_reciprocal=False):
     return codes, (amax / np.float32(448.0)).astype(np.float32)
 
 
+def swiglu(x, out_dtype="bf16"):
+    """[M, 2*I] float32 (values representable in out_dtype) -> [M, I] float32: silu(gate) * up with gate the
+    first half of a row and up the second, the product formed in fp32 and rounded once to out_dtype.
+    Defines the fused SwiGLU + quantisation operator of this build (no counterpart in the reference);
+    silu(x) = x / (1 + exp(-x)) with exp evaluated in float64 and rounded, i.e. the correctly rounded
+    fp32 exp that a device routine approximates to within an ulp or two."""
+    x = np.asarray(x, dtype=np.float32)
+    inter = x.shape[1] // 2
+    g, u = x[:, :inter], x[:, inter:]
+    e = np.exp(-g.astype(np.float64)).astype(np.float32)
+    h = ((g / (np.float32(1.0) + e)).astype(np.float32) * u).astype(np.float32)
+    return fp8.bf16_round(h) if out_dtype == "bf16" else fp8.fp16_round(h)
+
+
 def quant_weight_128x128(w, scale_via_reciprocal=False):
     """[N, K] float32 (both % 128 == 0) -> (codes uint8 [N, K], scales float32 [N/128, K/128]).
 

@@ -112,3 +112,48 @@ def test_quant_weight_bit_exact(esmoe, dtype, shape):
     assert torch.equal(q_o.view(torch.uint8), q_t.view(torch.uint8)) and torch.equal(sc_o, sc_t)
     assert torch.equal(q_o.view(torch.uint8), q)
     assert _native.lib.esmoe_fp8_quant_weight_128x128(ctypes.c_void_p(16), 0, ctypes.c_void_p(16), ctypes.c_void_p(16), 100, 128, None) == -1
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 128), (37, 384), (1030, 2048)])
+def test_swiglu_quant_against_oracle(esmoe, dtype, shape):
+    """Fused SwiGLU + 1x128 quantisation through the C ABI against oracle swiglu() -> quant_act_1x128().
+
+    Floating point with a transcendental: the device's fp32 exp is within an ulp or two of the oracle's
+    correctly rounded one, so a product that lands within that distance of a bf16/fp16 rounding boundary may
+    round the other way and move one byte (or, if it is the block maximum, the block's scale) by one step.
+    Tolerance: at most 1e-3 of the bytes and of the scales differ, and every dequantised value is within one
+    e4m3 step (12.5 % relative, plus the subnormal step) of the oracle's.  Zero products may carry either sign."""
+    from expert_specialization_moe_amd import _native
+    from oracle import fp8
+
+    m, inter = shape
+    gen = torch.Generator().manual_seed(m + inter)
+    x = (torch.randn((m, 2 * inter), generator=gen) * 2.0).to(dtype)
+    x[0, :8] = torch.tensor([-100.0, -20.0, 0.0, 20.0, 100.0, -0.0, 1e-3, -1e-3]).to(dtype)   # saturated and tiny gates
+    xd = x.cuda()
+    q = torch.full((m, inter), 0x55, dtype=torch.uint8, device="cuda")
+    sc = torch.full((m, inter // 128), -1.0, dtype=torch.float32, device="cuda")
+    rc = _native.lib.esmoe_swiglu_quant_1x128(H.ptr(xd), 0 if dtype == torch.bfloat16 else 1, H.ptr(q), H.ptr(sc), m, inter,
+                                              H.stream_ptr())
+    assert rc == 0, _native.last_error()
+    torch.cuda.synchronize()
+    with np.errstate(over="ignore"):
+        h = ofp8.swiglu(H.hp_to_f32(x), "bf16" if dtype == torch.bfloat16 else "fp16")
+    q_ref, sc_ref = ofp8.quant_act_1x128(h, scale_via_reciprocal=True)
+    qg, sg = q.cpu().numpy(), sc.cpu().numpy()
+    # the sign of a zero product (gate -0.0) is not pinned: 0x80 and 0x00 both decode to zero
+    canon = lambda c: np.where(c == 0x80, 0, c)
+    assert (canon(qg) != canon(q_ref)).mean() <= 1e-3, f"{(canon(qg) != canon(q_ref)).sum()} of {qg.size} bytes differ"
+    assert (sg != sc_ref).mean() <= 1e-3 + 1.0 / sg.size, f"{(sg != sc_ref).sum()} of {sg.size} scales differ"
+    deq_g = fp8.e4m3fn_decode(qg) * np.repeat(sg, 128, axis=1)
+    deq_r = fp8.e4m3fn_decode(q_ref) * np.repeat(sc_ref, 128, axis=1)
+    tol = 0.13 * np.abs(deq_r) + 1.1 * np.repeat(sc_ref, 128, axis=1) * 2.0 ** -9
+    assert (np.abs(deq_g - deq_r) <= tol).all()
+    # operator path gives the same bytes as the C ABI call
+    q_o, sc_o = esmoe.es_swiglu_quant_1x128(xd)
+    assert torch.equal(q_o.view(torch.uint8), q) and torch.equal(sc_o, sc)
+    # and stays close to the unfused torch sequence (two roundings instead of one)
+    hd = (torch.nn.functional.silu(xd[:, :inter].float()) * xd[:, inter:].float()).to(dtype)
+    q_t, sc_t = esmoe.es_fp8_quant_act_1x128(hd)
+    assert (q_t.view(torch.uint8) != q).float().mean().item() <= 2e-2

@@ -166,3 +166,25 @@ def test_quant_act_scale_variants_agree_within_one_ulp():
     d = np.abs(s0.view(np.int32).astype(np.int64) - s1.view(np.int32).astype(np.int64))
     assert d.max() <= 1 and (d == 1).any()
     assert np.array_equal(s1, s0 if False else (np.maximum(np.abs(x.reshape(64, 4, 128)).max(axis=2), np.float32(1e-4)) * (np.float32(1) / np.float32(448))).astype(np.float32))
+
+
+def test_swiglu_oracle_closed_forms():
+    """swiglu(): gate 0 -> 0; large positive gate -> gate * up; large negative gate -> (-)0; and agreement with a
+    float64 evaluation to one rounding of the output type."""
+    import numpy as np
+    from oracle import fp8
+    from oracle import fp8_blockwise as ofp8
+
+    x = np.array([[0.0, 30.0, -100.0, 1.5, 2.0, 0.5, 3.0, -2.0]], dtype=np.float32)   # gates | ups
+    with np.errstate(over="ignore"):
+        h = ofp8.swiglu(x)
+    assert h[0, 0] == 0.0 and h[0, 1] == 15.0 and h[0, 2] == 0.0
+    exact = 1.5 / (1.0 + np.exp(-1.5)) * -2.0
+    assert h[0, 3] == fp8.bf16_round(np.float32(exact))
+    rng = np.random.default_rng(3)
+    g = fp8.bf16_round(rng.standard_normal((16, 256)).astype(np.float32) * 3)
+    u = fp8.bf16_round(rng.standard_normal((16, 256)).astype(np.float32))
+    h = ofp8.swiglu(np.concatenate([g, u], axis=1))
+    ref = (g.astype(np.float64) / (1.0 + np.exp(-g.astype(np.float64)))) * u.astype(np.float64)
+    assert np.abs(h - ref).max() <= np.abs(ref).max() * 2.0 ** -8
+    assert (h == fp8.bf16_round(ref.astype(np.float32))).mean() > 0.999
