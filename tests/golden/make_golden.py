@@ -8,6 +8,9 @@ project's own known-answer vectors:
   mx_quant_small.npz     a ragged MXFP8 grouped-quant case: bf16 input bits, expected e4m3 bytes,
                          swizzled E8M0 scale bytes and the mask of defined scale bytes
   sf_swizzle_table.npz   byte offsets of the swizzled scale layout for M in {1,127,128,129,300}, K in {128,384}
+  caller_side_small.npz  the caller-side steps on a 40-token, top-2, 6-expert case (ids 0..7, so two experts are
+                         remote): routing metadata and packing order, packed bf16 rows, their 1x128 quantisation
+                         (scale = amax * fl(1/448), the GPU flavour) and a 128x128 weight quantisation
 
 Run from the repository root:  python tests/golden/make_golden.py
 """
@@ -20,6 +23,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)
 sys.path.insert(0, ROOT)
 from oracle import fp8, mxfp8  # noqa: E402
 from oracle import fp8_blockwise as ofp8  # noqa: E402
+from oracle import routing as oroute  # noqa: E402
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -69,7 +73,25 @@ def sf_table():
     np.savez_compressed(os.path.join(HERE, "sf_swizzle_table.npz"), **out)
 
 
+def caller_side():
+    rng = np.random.default_rng(2)
+    tokens, topk, experts, k = 40, 2, 6, 256
+    ids = np.stack([rng.permutation(8)[:topk] for _ in range(tokens)]).astype(np.int32)
+    x = fp8.bf16_round((rng.standard_normal((tokens, k)) * np.exp(rng.uniform(-3, 3, (tokens, 1)))).astype(np.float32))
+    x[5, :128] = 0.0
+    ps, eo, bso, dst = oroute.route_metadata(ids, 0, experts, 128, k)
+    packed = oroute.permute_rows(x, dst, topk, int(eo[-1]))
+    q, sc = ofp8.quant_act_1x128(packed, scale_via_reciprocal=True)
+    w = fp8.bf16_round((rng.standard_normal((128, k)) * 0.03).astype(np.float32))
+    wq, wsc = ofp8.quant_weight_128x128(w, scale_via_reciprocal=True)
+    np.savez_compressed(os.path.join(HERE, "caller_side_small.npz"), topk_ids=ids, x_bf16_bits=fp8.bf16_bits(x),
+                        problem_sizes=ps, expert_offsets=eo, blockscale_offsets=bso, dst_row=dst,
+                        packed_bf16_bits=fp8.bf16_bits(packed), q=q, scales=sc, w_bf16_bits=fp8.bf16_bits(w), wq=wq,
+                        wscales=wsc)
+
+
 if __name__ == "__main__":
+    caller_side()
     c0()
     mx_quant()
     sf_table()

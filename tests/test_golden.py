@@ -67,3 +67,37 @@ def test_gpu_matches_quant_fixture_bit_exact(esmoe):
     torch.cuda.synchronize()
     assert np.array_equal(q.cpu().numpy(), g["q"])
     assert np.array_equal(sf.cpu().numpy()[g["sf_mask"]], g["sf"][g["sf_mask"]])
+
+
+def test_oracle_reproduces_caller_side_fixture():
+    from oracle import routing as oroute
+
+    g = np.load(os.path.join(GOLD, "caller_side_small.npz"))
+    ids, x = g["topk_ids"], fp8.bf16_from_bits(g["x_bf16_bits"])
+    ps, eo, bso, dst = oroute.route_metadata(ids, 0, 6, 128, x.shape[1])
+    assert np.array_equal(ps, g["problem_sizes"]) and np.array_equal(eo, g["expert_offsets"])
+    assert np.array_equal(bso, g["blockscale_offsets"]) and np.array_equal(dst, g["dst_row"])
+    packed = oroute.permute_rows(x, dst, ids.shape[1], int(eo[-1]))
+    assert np.array_equal(fp8.bf16_bits(packed), g["packed_bf16_bits"])
+    q, sc = ofp8.quant_act_1x128(packed, scale_via_reciprocal=True)
+    assert np.array_equal(q, g["q"]) and np.array_equal(sc, g["scales"])
+    wq, wsc = ofp8.quant_weight_128x128(fp8.bf16_from_bits(g["w_bf16_bits"]), scale_via_reciprocal=True)
+    assert np.array_equal(wq, g["wq"]) and np.array_equal(wsc, g["wscales"])
+
+
+@pytest.mark.gpu
+def test_gpu_matches_caller_side_fixture_bit_exact(esmoe):
+    g = np.load(os.path.join(GOLD, "caller_side_small.npz"))
+    ids = torch.from_numpy(g["topk_ids"]).cuda()
+    x = torch.from_numpy(g["x_bf16_bits"].astype(np.int16)).view(torch.bfloat16).cuda()
+    ps, eo, bso, dst = esmoe.es_route_metadata(ids, 0, 6, 128, x.shape[1])
+    assert np.array_equal(ps.cpu().numpy(), g["problem_sizes"]) and np.array_equal(eo.cpu().numpy(), g["expert_offsets"])
+    assert np.array_equal(bso.cpu().numpy(), g["blockscale_offsets"]) and np.array_equal(dst.cpu().numpy(), g["dst_row"])
+    packed = torch.zeros((int(g["expert_offsets"][-1]), x.shape[1]), dtype=torch.bfloat16, device="cuda")
+    esmoe.es_permute_rows(x, dst, ids.shape[1], packed)
+    assert np.array_equal(packed.view(torch.int16).cpu().numpy().view(np.uint16), g["packed_bf16_bits"])
+    q, sc = esmoe.es_fp8_quant_act_1x128(packed)
+    assert np.array_equal(q.view(torch.uint8).cpu().numpy(), g["q"]) and np.array_equal(sc.cpu().numpy(), g["scales"])
+    w = torch.from_numpy(g["w_bf16_bits"].astype(np.int16)).view(torch.bfloat16).cuda()
+    wq, wsc = esmoe.es_fp8_quant_weight_128x128(w)
+    assert np.array_equal(wq.view(torch.uint8).cpu().numpy(), g["wq"]) and np.array_equal(wsc.cpu().numpy(), g["wscales"])
