@@ -275,7 +275,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     v8i af[kPre];
     int sfw[MX ? NTW : 1];
     int sfa[MX ? MTW : 1];
-    float sc[MX ? 1 : MTW];
+    float sc[MX ? 1 : MTW];   // fp8-blockwise: sa of the row tiles (the product with sb is formed in the mfma phase)
+    float sb;
   };
 
   auto read_phase = [&](int kb, int buf, Frags& f) {
@@ -314,19 +315,54 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
         f.sfa[mt] = (int)(d >> (gq * 8));
       }
     } else {
-      const float sbv = sb_tab[kb];
+      f.sb = sb_tab[kb];
 #pragma unroll
       for (int mt = 0; mt < MTW; mt++) {
-        f.sc[mt] = (sa4 ? *(const float*)(lds + sa4_lane + ((kb >> 2) & 1) * 4096 + (kb & 3) * 4 + mt * 256)
-                        : *(const float*)(lb + sa_lane + mt * 64)) * sbv;
+        f.sc[mt] = sa4 ? *(const float*)(lds + sa4_lane + ((kb >> 2) & 1) * 4096 + (kb & 3) * 4 + mt * 256)
+                       : *(const float*)(lb + sa_lane + mt * 64);
       }
     }
   };
 
-  // The fp32 promotion of row tile mt runs behind the MFMAs of row tile mt + 1, so that the vector ALU
-  // works in the shadow of the matrix pipe.
+  // fp8-blockwise with all fragments in registers: MFMAs and promotions form one scheduling region in which
+  // the four v_fmac of MFMA j - 3 follow MFMA j, so the vector ALU works in the shadow of the matrix pipe
+  // and no promotion waits on the MFMA it has just been issued behind.  Taller tiles (fragments read from
+  // LDS during the phase) keep the coarser order: promotion of row tile mt behind the MFMAs of mt + 1.
   auto mfma_phase = [&](int buf, const Frags& f) {
     const uint8_t* lb = lds + buf * G::kStageBytes;
+    if constexpr (!MX && kPre == MTW) {
+      // all fragments are in registers: one scheduling region in which promotion j - LAG issues behind MFMA j
+      float sc[MTW];
+#pragma unroll
+      for (int mt = 0; mt < MTW; mt++) sc[mt] = f.sc[mt] * f.sb;
+      v4f t[MTW][NTW];
+#pragma unroll
+      for (int mt = 0; mt < MTW; mt++)
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++)
+          t[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], f.af[mt], v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+      for (int mt = 0; mt < MTW; mt++)
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) acc[nt][mt][i] = __builtin_fmaf(t[mt][nt][i], sc[mt], acc[nt][mt][i]);
+      constexpr int kT = MTW * NTW, kLag = 3;
+#pragma unroll
+      for (int j = 0; j < kLag; j++) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+      for (int j = kLag; j < kT; j++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < kLag; j++) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+#pragma unroll
+      for (int mt = 0; mt < MTW; mt++)
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) asm volatile("" : "+v"(acc[nt][mt]));   // the promotions stay in this phase
+      return;
+    }
     v4f tmp[2][NTW];
 #pragma unroll
     for (int mt = 0; mt < MTW; mt++) {
@@ -350,7 +386,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
           for (int nt = 0; nt < NTW; nt++) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[nt][mt - 1][i] = __builtin_fmaf(tmp[(mt - 1) & 1][nt][i], f.sc[mt - 1], acc[nt][mt - 1][i]);
+            for (int i = 0; i < 4; i++) acc[nt][mt - 1][i] = __builtin_fmaf(tmp[(mt - 1) & 1][nt][i], f.sc[mt - 1] * f.sb, acc[nt][mt - 1][i]);
             asm volatile("" : "+v"(acc[nt][mt - 1]));  // keeps the promotion here, in the shadow of the MFMAs above
           }
         }
@@ -361,7 +397,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
       for (int nt = 0; nt < NTW; nt++) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[nt][MTW - 1][i] = __builtin_fmaf(tmp[(MTW - 1) & 1][nt][i], f.sc[MTW - 1], acc[nt][MTW - 1][i]);
+        for (int i = 0; i < 4; i++) acc[nt][MTW - 1][i] = __builtin_fmaf(tmp[(MTW - 1) & 1][nt][i], f.sc[MTW - 1] * f.sb, acc[nt][MTW - 1][i]);
         asm volatile("" : "+v"(acc[nt][MTW - 1]));
       }
     }
@@ -391,14 +427,18 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // Barrier intervals alternate; group 0 (wavefronts 0-3) reads K block kb in interval 2kb and runs its
   // MFMAs in interval 2kb+1, group 1 (wavefronts 4-7) does each one interval later.  Ring slot of K
   // block kb is therefore read during intervals 2kb and 2kb+1 and must be complete before interval
-  // 2kb starts; it is refilled with K block kb+NBUF from interval 2kb+2 on: by group 1 at the start of
-  // its mfma phase kb (interval 2kb+2), by group 0 at the start of its mfma phase kb+1 (interval 2kb+3).
-  // Issuing the copies costs a wavefront a few hundred cycles; putting them in front of the MFMAs
-  // evens out the two groups' phases (the read phase waits on LDS latency already).
+  // 2kb starts; it is refilled with K block kb+NBUF from interval 2kb+2 on (each group's read phase
+  // kb+1; for mxfp8 the weight rows a phase later, see kSplitIssue).  Issuing copies costs a wavefront
+  // a few hundred cycles in the queue to the texture path, so where they sit decides which phase is
+  // the longer one.
   // Tiles whose mfma phase still reads token fragments from LDS (16 row tiles per wavefront do not
   // fit in registers) run both groups in step, with no barrier between the phases.
   constexpr bool kPP = kPre == MTW;
   const int grp = kPP ? wave >> 2 : 0;
+  // mxfp8 (no vector-ALU work in the mfma phase): token copies go out in the read phase, weight copies in
+  // the mfma phase.  fp8-blockwise: the mfma phase is already the longer one with its promotions, so
+  // the read phase issues the whole stage.
+  constexpr bool kSplitIssue = kPP && MX;
   auto wait_stage = [&](bool more, int chunk_young) {
     // all of this wavefront's copies except those of the newest NBUF-2 K blocks have landed
     if (!more) wait_vmcnt<0>();
@@ -409,7 +449,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   int buf = 0, nbuf = NBUF - 1;  // ring slots of K block kb and of K block kb + NBUF - 1
   int chunk_age = NBUF;          // iterations since this wavefront issued a scale-chunk copy
   if (grp == 1) {
-    if (NBUF - 1 < KB) issue_w(NBUF - 1, nbuf);
+    if constexpr (kSplitIssue) { if (NBUF - 1 < KB) issue_w(NBUF - 1, nbuf); }
     block_barrier();
   }
   Frags f;
@@ -422,13 +462,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       issue_sa_chunk((kb >> 2) + 1);
       chunk_age = 0;
     }
-    if (more) { if constexpr (kPP) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
+    if (more) { if constexpr (kSplitIssue) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
     __builtin_amdgcn_sched_barrier(0);
     read_phase(kb, buf, f);
     __builtin_amdgcn_sched_barrier(0);
     if (grp == 1) wait_stage(more, chunk_age < NBUF - 2);
     if constexpr (kPP) block_barrier();
-    if constexpr (kPP) {
+    if constexpr (kSplitIssue) {
       if (grp == 0) { if (more) issue_w(kb + NBUF - 1, nbuf); }
       else if (kb + NBUF < KB) issue_w(kb + NBUF, buf);
     }
