@@ -20,8 +20,8 @@ import torch
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "gemm"): 1.638e9,     # FETCH 773,495.5 x 2.000 KiB + WRITE 52,929.4 x 1.000 KiB
-    ("c4", "quant"): 1.786e8,    # FETCH 57,398.6 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
+    ("c1", "gemm"): 1.634e9,     # FETCH 771,376.7 x 2.000 KiB + WRITE 53,101.0 x 1.000 KiB
+    ("c4", "quant"): 1.786e8,    # FETCH 57,398.5 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
 }
 
 
