@@ -58,8 +58,10 @@ lib.esmoe_version.restype = ctypes.c_char_p
 lib.esmoe_version.argtypes = []
 lib.esmoe_host_schedule.restype = _i
 lib.esmoe_host_schedule.argtypes = [_vp, _i, _i, _i, _vp]
-lib.esmoe_host_decode_item.restype = _i
-lib.esmoe_host_decode_item.argtypes = [_vp, _vp, _i, _i, _i, _i, _vp]
+lib.esmoe_host_decode_heavy.restype = _i
+lib.esmoe_host_decode_heavy.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
+lib.esmoe_host_decode_light.restype = _i
+lib.esmoe_host_decode_light.argtypes = [_vp, _vp, _i, _i, _i, _i, _vp]
 
 
 def last_error():

@@ -89,6 +89,7 @@ esmoe::SchedPolicy make_policy(int force_bm, int mx) {
   // 192 rows, and shorter full tiles leave less padding in the remainder tile.
   p.big_mt = env_int("ESMOE_BIG_MT", mx ? 16 : 12);
   p.order = env_int("ESMOE_ORDER", 0);
+  p.light_share = env_int("ESMOE_LIGHT_SHARE", -1);
   return p;
 }
 
@@ -310,49 +311,82 @@ int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int 
   if (!problem_sizes_host || !ws_host || num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS || n <= 0 || n % 128)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_schedule");
   const esmoe::SchedPolicy p = make_policy(force_bm, 0);
-  int32_t* item_start = ws_host + esmoe::ws_item_start(num_experts);
-  int32_t* order = ws_host + esmoe::ws_order(num_experts);
+  auto rows_of = [&](int e) { return problem_sizes_host[e * 3] < 0 ? 0 : problem_sizes_host[e * 3]; };
   // same ranking as the device schedule kernel: most rows first, ties by expert index
   for (int e = 0; e < num_experts; e++) {
-    int m = problem_sizes_host[e * 3] < 0 ? 0 : problem_sizes_host[e * 3];
     int pos = e;
     if (p.order == 0) {
       pos = 0;
-      for (int j = 0; j < num_experts; j++) {
-        int mj = problem_sizes_host[j * 3] < 0 ? 0 : problem_sizes_host[j * 3];
-        pos += (mj > m) || (mj == m && j < e);
-      }
+      for (int j = 0; j < num_experts; j++) pos += (rows_of(j) > rows_of(e)) || (rows_of(j) == rows_of(e) && j < e);
     }
-    order[pos] = e;
+    ws_host[esmoe::ws_rec(pos) + esmoe::kRecExpert] = e;
+    ws_host[esmoe::ws_rec(pos) + esmoe::kRecRows] = rows_of(e);
   }
-  int run = 0;
+  int blocks = 0, items = 0;
+  long heavy_cost = 0, light_cost = 0;
   for (int pos = 0; pos < num_experts; pos++) {
-    int m = problem_sizes_host[order[pos] * 3];
-    item_start[pos] = run;
-    run += esmoe::sched_items(m, n, p);
+    const int m = ws_host[esmoe::ws_rec(pos) + esmoe::kRecRows];
+    ws_host[esmoe::ws_rec(pos) + esmoe::kRecBlock] = blocks;
+    ws_host[esmoe::ws_rec(pos) + esmoe::kRecItem] = items;
+    blocks += esmoe::sched_heavy_blocks(m, n, p);
+    items += esmoe::sched_light_items(m, n, p);
+    heavy_cost += esmoe::sched_heavy_cost(m, n, p);
+    light_cost += esmoe::sched_light_cost(m, n, p);
   }
-  item_start[num_experts] = run;
-  ws_host[esmoe::kWsTotal] = run;
-  ws_host[esmoe::kWsCounter] = 0;
+  int32_t* last = ws_host + esmoe::ws_rec(num_experts);
+  last[esmoe::kRecBlock] = blocks;
+  last[esmoe::kRecItem] = items;
+  last[esmoe::kRecExpert] = -1;
+  last[esmoe::kRecRows] = 0;
+  ws_host[esmoe::kWsLightShare] = esmoe::sched_light_share(heavy_cost, light_cost, p);
+  ws_host[esmoe::kWsHeavyBlocks] = blocks;
+  ws_host[esmoe::kWsLightTotal] = items;
+  ws_host[esmoe::kWsLightCounter] = 0;
+  for (int x = 0; x < esmoe::kXcds; x++) ws_host[esmoe::kWsXcdCounter + x] = 0;
   return 0;
 }
 
-int esmoe_host_decode_item(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                           int force_bm, int item, int32_t* out5) {
+namespace {
+// Schedule position whose [first, next) range of blocks (kind kRecBlock) or items (kRecItem) holds v.
+int host_position(const int32_t* ws_host, int num, int kind, int v) {
+  for (int pos = 0; pos < num; pos++)
+    if (ws_host[esmoe::ws_rec(pos) + kind] <= v && v < ws_host[esmoe::ws_rec(pos + 1) + kind]) return pos;
+  return -1;
+}
+void fill_out5(int32_t* out5, int e, const esmoe::TileCoord& t) {
+  out5[0] = e; out5[1] = t.mt * 16; out5[2] = t.nt * 64; out5[3] = t.m0; out5[4] = t.n0;
+}
+}  // namespace
+
+int esmoe_host_decode_heavy(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
+                            int force_bm, int xcd, int ticket, int32_t* out5) {
+  g_err[0] = 0;
+  if (!problem_sizes_host || !ws_host || !out5 || xcd < 0 || xcd >= esmoe::kXcds || ticket < 0)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_decode_heavy");
+  const esmoe::SchedPolicy p = make_policy(force_bm, 0);
+  const int blk = esmoe::sched_ticket_block(xcd, ticket);
+  if (blk >= ws_host[esmoe::kWsHeavyBlocks]) return 2;   // this XCD's queue is exhausted
+  const int pos = host_position(ws_host, num_experts, esmoe::kRecBlock, blk);
+  if (pos < 0) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace does not hold a schedule");
+  const int32_t* rec = ws_host + esmoe::ws_rec(pos);
+  esmoe::TileCoord t;
+  if (!esmoe::sched_decode_heavy(blk - rec[esmoe::kRecBlock], ticket % esmoe::kBlkTiles, rec[esmoe::kRecRows], n, p, &t))
+    return 1;   // ticket outside the expert's tile grid: skipped
+  fill_out5(out5, rec[esmoe::kRecExpert], t);
+  return 0;
+}
+
+int esmoe_host_decode_light(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
+                            int force_bm, int item, int32_t* out5) {
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || !out5) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null pointer");
+  (void)n;
   const esmoe::SchedPolicy p = make_policy(force_bm, 0);
-  const int32_t* item_start = ws_host + esmoe::ws_item_start(num_experts);
-  const int32_t* order = ws_host + esmoe::ws_order(num_experts);
-  if (item < 0 || item >= ws_host[esmoe::kWsTotal]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "item out of range");
-  int lo = 0, hi = num_experts;
-  while (hi - lo > 1) {
-    int mid = (lo + hi) >> 1;
-    if (item_start[mid] <= item) lo = mid; else hi = mid;
-  }
-  const int e = order[lo];
-  const esmoe::TileCoord t = esmoe::sched_decode(item - item_start[lo], problem_sizes_host[e * 3], n, p);
-  out5[0] = e; out5[1] = t.mt * 16; out5[2] = t.nt * 64; out5[3] = t.m0; out5[4] = t.n0;
+  if (item < 0 || item >= ws_host[esmoe::kWsLightTotal]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "item out of range");
+  const int pos = host_position(ws_host, num_experts, esmoe::kRecItem, item);
+  if (pos < 0) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace does not hold a schedule");
+  const int32_t* rec = ws_host + esmoe::ws_rec(pos);
+  fill_out5(out5, rec[esmoe::kRecExpert], esmoe::sched_decode_light(item - rec[esmoe::kRecItem], rec[esmoe::kRecRows], p));
   return 0;
 }
 

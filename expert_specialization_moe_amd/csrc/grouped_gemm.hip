@@ -506,19 +506,20 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 
 // ---------------------------------------------------------------------------------------------
 // Schedule kernel: one workgroup, thread = expert (E <= 1024, as the reference's pre-compute kernel,
-// es_fp8_blockwise_launcher.cuh:53,74).
+// es_fp8_blockwise_launcher.cuh:53,74).  Ranks the experts by rows (most first), prefix-sums the heavy
+// experts' tile blocks and the light experts' items over that order, and zeroes the hand-out counters.
 __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ problem_sizes, int num_experts, int n,
                                                         SchedPolicy policy, int* __restrict__ ws) {
   __shared__ int s_m[1024];
+  __shared__ int s_blocks[1024];
   __shared__ int s_items[1024];
+  __shared__ long s_cost[1024][2];
   const int e = threadIdx.x;
   int m = 0;
   if (e < num_experts) m = problem_sizes[e * 3];
   if (m < 0) m = 0;
   s_m[e] = m;
   __syncthreads();
-  int* item_start = ws + ws_item_start(num_experts);
-  int* order = ws + ws_order(num_experts);
   int pos = e;
   if (e < num_experts) {
     if (policy.order == 0) {
@@ -528,22 +529,43 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
         pos += (mj > m) || (mj == m && j < e);
       }
     }
-    order[pos] = e;
-    s_items[pos] = sched_items(m, n, policy);
+    ws[ws_rec(pos) + kRecExpert] = e;
+    ws[ws_rec(pos) + kRecRows] = m;
+    s_blocks[pos] = sched_heavy_blocks(m, n, policy);
+    s_items[pos] = sched_light_items(m, n, policy);
+    s_cost[pos][0] = sched_heavy_cost(m, n, policy);
+    s_cost[pos][1] = sched_light_cost(m, n, policy);
   }
   __syncthreads();
   if (e < num_experts) {
-    // exclusive prefix sum over schedule positions, one position per thread
-    int run = 0;
-    for (int j = 0; j < pos; j++) run += s_items[j];
-    item_start[pos] = run;
-    if (pos == num_experts - 1) {
-      run += s_items[pos];
-      item_start[num_experts] = run;
-      ws[kWsTotal] = run;
-      ws[kWsCounter] = 0;
+    // exclusive prefix sums over schedule positions, one position per thread
+    int blocks = 0, items = 0;
+    for (int j = 0; j < pos; j++) {
+      blocks += s_blocks[j];
+      items += s_items[j];
     }
+    ws[ws_rec(pos) + kRecBlock] = blocks;
+    ws[ws_rec(pos) + kRecItem] = items;
+    if (pos == num_experts - 1) {
+      blocks += s_blocks[pos];
+      items += s_items[pos];
+      ws[ws_rec(num_experts) + kRecBlock] = blocks;
+      ws[ws_rec(num_experts) + kRecItem] = items;
+      ws[ws_rec(num_experts) + kRecExpert] = -1;
+      ws[ws_rec(num_experts) + kRecRows] = 0;
+      ws[kWsHeavyBlocks] = blocks;
+      ws[kWsLightTotal] = items;
+      ws[kWsLightCounter] = 0;
+      long heavy_cost = 0, light_cost = 0;
+      for (int j = 0; j < num_experts; j++) {
+        heavy_cost += s_cost[j][0];
+        light_cost += s_cost[j][1];
+      }
+      ws[kWsLightShare] = sched_light_share(heavy_cost, light_cost, policy);
+    }
+    if (pos < kXcds) ws[kWsXcdCounter + pos] = 0;
   }
+  if (num_experts < kXcds && e >= num_experts && e < kXcds) ws[kWsXcdCounter + e] = 0;
 }
 
 // Tile heights (MT * 16 rows) compiled into the persistent kernel.
@@ -555,34 +577,85 @@ template <bool MX>
 __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
   __shared__ int s_item;
+  __shared__ int s_rec[3];   // expert, its rows, index of the block or item inside the expert
   int* ws = g.ws;
-  const int total = ws[kWsTotal];
-  const int* item_start = ws + ws_item_start(g.num_experts);
-  const int* order = ws + ws_order(g.num_experts);
-  for (;;) {
-    if (threadIdx.x == 0) s_item = atomicAdd(&ws[kWsCounter], 1);
-    __syncthreads();
-    const int item = __builtin_amdgcn_readfirstlane(s_item);
-    __syncthreads();
-    if (item >= total) break;
-    // position p with item_start[p] <= item < item_start[p+1]
-    int lo = 0, hi = g.num_experts;
-    while (hi - lo > 1) {
-      int mid = (lo + hi) >> 1;
-      if (item_start[mid] <= item) lo = mid; else hi = mid;
-    }
-    const int e = order[lo];
-    const int M = g.problem_sizes[e * 3];
-    const TileCoord t = sched_decode(item - item_start[lo], M, g.n, g.policy);
-    const int key = t.mt;
+  const int hblocks = ws[kWsHeavyBlocks];
+  const int ltotal = ws[kWsLightTotal];
 #define ESMOE_CASE(MT_) \
   case (MT_): gemm_tile<MT_, MX>(g, e, M, t.m0, t.n0, lds); break;
-    switch (key) {
+
+  // Workgroup i runs on XCD i % 8 (HW_REG_XCC_ID = 20, bits [3:0], says so directly).  Of every 32 workgroups
+  // of an XCD the last `light_share` start on the light items, the others on the heavy tickets; either kind
+  // moves on to the other when its own is exhausted.
+  const int xcd = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & (kXcds - 1);
+  const int per_xcd = (int)gridDim.x / kXcds > 0 ? (int)gridDim.x / kXcds : 1;
+  const bool light_first = (int)(blockIdx.x / kXcds) * 32 / per_xcd >= 32 - ws[kWsLightShare];
+  int phase = 0, q = 0;
+#ifdef ESMOE_TIMELINE
+  int tl_n = 0;
+  if (threadIdx.x == 0) ((uint32_t*)ws)[4096 + blockIdx.x * 128] = 0;
+#endif
+  for (;;) {
+    const bool light = (phase == 0) == light_first;
+    const int xq = (xcd + q) & (kXcds - 1);
+    if (light ? ltotal == 0 : xq >= hblocks) {   // nothing of this kind (or this queue never had a block)
+      if (light || ++q == kXcds) {
+        q = 0;
+        if (++phase == 2) break;
+      }
+      continue;
+    }
+    if (threadIdx.x == 0) s_item = atomicAdd(light ? &ws[kWsLightCounter] : &ws[kWsXcdCounter + xq], 1);
+    __syncthreads();
+    const int ticket = __builtin_amdgcn_readfirstlane(s_item);
+    // every thread tests one schedule position (two beyond 512 experts) against the prefix sums: one
+    // round trip to memory instead of a dependent search
+    const int kind = light ? kRecItem : kRecBlock;
+    const int v = light ? ticket : sched_ticket_block(xq, ticket);
+    if (v >= (light ? ltotal : hblocks)) {   // this queue is exhausted: the next XCD's, then the other kind
+      __syncthreads();                        // s_item is rewritten next
+      if (light || ++q == kXcds) {
+        q = 0;
+        if (++phase == 2) break;
+      }
+      continue;
+    }
+    for (int i = threadIdx.x; i < g.num_experts; i += kThreads) {
+      const int* rec = ws + ws_rec(i);
+      const int first = rec[kind], next = rec[kRecWords + kind], re = rec[kRecExpert], rm = rec[kRecRows];
+      if (first <= v && v < next) {
+        s_rec[0] = re;
+        s_rec[1] = rm;
+        s_rec[2] = v - first;
+      }
+    }
+    __syncthreads();
+    const int e = __builtin_amdgcn_readfirstlane(s_rec[0]), M = __builtin_amdgcn_readfirstlane(s_rec[1]);
+    const int local = __builtin_amdgcn_readfirstlane(s_rec[2]);
+    TileCoord t;
+    if (light) t = sched_decode_light(local, M, g.policy);
+    else if (!sched_decode_heavy(local, ticket % kBlkTiles, M, g.n, g.policy, &t)) continue;
+#ifdef ESMOE_TIMELINE
+    const uint64_t tl_t0 = __builtin_amdgcn_s_memrealtime();
+#endif
+    switch (t.mt) {
       ESMOE_VARIANTS
       default: break;
     }
-#undef ESMOE_CASE
+#ifdef ESMOE_TIMELINE
+    // debug build only: (start, end, kind) of this workgroup's first 31 tiles, in 100 MHz ticks, into a
+    // caller-provided oversize workspace from word 4096 on
+    if (threadIdx.x == 0 && tl_n < 31) {
+      uint32_t* tl = (uint32_t*)ws + 4096 + blockIdx.x * 128;
+      tl[4 + tl_n * 4 + 0] = (uint32_t)tl_t0;
+      tl[4 + tl_n * 4 + 1] = (uint32_t)__builtin_amdgcn_s_memrealtime();
+      tl[4 + tl_n * 4 + 2] = (uint32_t)(t.mt | (light ? 256 : 0) | (xcd << 12) | (e << 16));
+      tl[4 + tl_n * 4 + 3] = (uint32_t)(t.m0 / 16) | ((uint32_t)(t.n0 / 256) << 16);
+      tl[0] = ++tl_n;
+    }
+#endif
   }
+#undef ESMOE_CASE
 }
 
 }  // namespace esmoe

@@ -27,6 +27,7 @@ struct SchedPolicy {
   int force_mt;   // 0 = choose per expert; else every tile uses this MT
   int big_mt;     // MT of the full tiles of a many-row expert (8, 12 or 16)
   int order;      // 0: experts sorted by rows, most rows first; 1: expert index order
+  int light_share;  // workgroups (of every 32) that start on the light items; -1 = from the cost estimate
 };
 
 struct TileCoord {
@@ -53,62 +54,118 @@ ESMOE_HD int sched_nt_for(int, const SchedPolicy&) { return 4; }
 
 ESMOE_HD int sched_ntiles(int n, int nt) { return (n + nt * 64 - 1) / (nt * 64); }
 
-// Number of work items of an expert with `m` rows and `n` columns.
-ESMOE_HD int sched_items(int m, int n, const SchedPolicy& p) {
-  if (m <= 0) return 0;
-  if (p.force_mt) {
-    int rows = p.force_mt * 16;
-    return ((m + rows - 1) / rows) * sched_ntiles(n, sched_nt_for(p.force_mt, p));
-  }
-  int big_rows = p.big_mt * 16;
-  int full = m / big_rows;
-  int rem = m - full * big_rows;
-  int items = full * sched_ntiles(n, sched_nt_for(p.big_mt, p));
-  if (rem) {
-    int rmt = sched_cover_mt(rem, p.big_mt);
-    items += sched_ntiles(n, sched_nt_for(rmt, p));
-  }
-  return items;
+// ---- XCD-aware hand-out ------------------------------------------------------------------
+// The 256 CUs sit in 8 XCDs with one L2 each, and workgroup i of a launch runs on XCD i % 8.  Tiles
+// of one expert that share token rows or weight rows should therefore run at the same time on the
+// same XCD: every expert with more than 64 rows ("heavy") has its tile grid cut into blocks of
+// up to 32 tiles (one per CU of an XCD, at most kBlkM tiles high), block b of the launch belongs to XCD b % 8, and the
+// workgroups of an XCD draw tickets from that XCD's counter: ticket t is tile t % 32 of the XCD's
+// (t / 32)-th block.  A dense 6144 x 4096 x 7168 problem fetches 302 MB into L2 this way against
+// 557 MB with tiles handed out in plain order.  Tickets that fall outside the grid (edge blocks) are
+// skipped.  An XCD that runs out of blocks helps the others.  Experts with at most 64 rows ("light")
+// have one short tile per 256 columns that streams its weights once; nothing is shared, and they come
+// from one launch-wide counter.  Heavy tiles are bound by the LDS feed of the matrix cores and light
+// items by HBM, so the two kinds run side by side: a share of the workgroups (sized by the cost
+// estimates below) starts on the light items while the rest start on the heavy tickets, and each
+// side moves on to the other kind when its own runs out.
+constexpr int kBlkM = 8;
+constexpr int kBlkTiles = 32;
+constexpr int kXcds = 8;
+
+ESMOE_HD bool sched_is_heavy(int m, const SchedPolicy& p) { return p.force_mt ? m > 0 : m > 64; }
+
+// Row tiles of an expert: full big tiles plus one remainder tile.
+ESMOE_HD int sched_mtiles(int m, const SchedPolicy& p) {
+  const int rows = (p.force_mt ? p.force_mt : p.big_mt) * 16;
+  return (m + rows - 1) / rows;
 }
 
-// Inverse of the enumeration counted by sched_items: column tiles vary fastest,
-// full row tiles come first, the remainder tile last.
-ESMOE_HD TileCoord sched_decode(int item, int m, int n, const SchedPolicy& p) {
+// Block shape for an expert with mtl x ntl tiles: at most kBlkM tiles high and kBlkTiles tiles in all, with
+// the rows and the columns of the grid split evenly over the blocks (21 x 16 tiles -> blocks of 7 x 4;
+// 6 x 16 -> 6 x 4; 1 x 16 -> 1 x 16).  Near-square blocks (in bytes) fetch the least per tile.
+ESMOE_HD void sched_block_shape(int mtl, int ntl, int* bm, int* bn) {
+  const int rb = (mtl + kBlkM - 1) / kBlkM;
+  *bm = (mtl + rb - 1) / rb;
+  const int w = kBlkTiles / *bm;
+  const int cb = (ntl + w - 1) / w;
+  *bn = (ntl + cb - 1) / cb;
+}
+
+ESMOE_HD int sched_heavy_blocks(int m, int n, const SchedPolicy& p) {
+  if (!sched_is_heavy(m, p)) return 0;
+  const int mtl = sched_mtiles(m, p), ntl = sched_ntiles(n, 4);
+  int bm, bn;
+  sched_block_shape(mtl, ntl, &bm, &bn);
+  return ((mtl + bm - 1) / bm) * ((ntl + bn - 1) / bn);
+}
+
+ESMOE_HD int sched_light_items(int m, int n, const SchedPolicy& p) {
+  return (m > 0 && !sched_is_heavy(m, p)) ? sched_ntiles(n, 4) : 0;
+}
+
+// Tile `idx` (0..31) of block `lb` of a heavy expert; false if it falls outside the expert's grid.
+ESMOE_HD bool sched_decode_heavy(int lb, int idx, int m, int n, const SchedPolicy& p, TileCoord* t) {
+  const int mtl = sched_mtiles(m, p), ntl = sched_ntiles(n, 4);
+  int bm, bn;
+  sched_block_shape(mtl, ntl, &bm, &bn);
+  const int nbc = (ntl + bn - 1) / bn;
+  if (idx >= bm * bn) return false;
+  const int mi = (lb / nbc) * bm + idx / bn, ni = (lb % nbc) * bn + idx % bn;
+  if (mi >= mtl || ni >= ntl) return false;
+  const int big = p.force_mt ? p.force_mt : p.big_mt;
+  const int m0 = mi * big * 16;
+  t->mt = p.force_mt ? p.force_mt : (m - m0 >= big * 16 ? big : sched_cover_mt(m - m0, big));
+  t->nt = 4;
+  t->m0 = m0;
+  t->n0 = ni * 256;
+  return true;
+}
+
+ESMOE_HD TileCoord sched_decode_light(int item, int m, const SchedPolicy& p) {
   TileCoord t;
-  if (p.force_mt) {
-    t.mt = p.force_mt;
-    t.nt = sched_nt_for(t.mt, p);
-    int ntl = sched_ntiles(n, t.nt);
-    t.m0 = (item / ntl) * t.mt * 16;
-    t.n0 = (item % ntl) * t.nt * 64;
-    return t;
-  }
-  int big_rows = p.big_mt * 16;
-  int full = m / big_rows;
-  int nt_big = sched_nt_for(p.big_mt, p);
-  int ntl_big = sched_ntiles(n, nt_big);
-  int full_items = full * ntl_big;
-  if (item < full_items) {
-    t.mt = p.big_mt;
-    t.nt = nt_big;
-    t.m0 = (item / ntl_big) * big_rows;
-    t.n0 = (item % ntl_big) * nt_big * 64;
-    return t;
-  }
-  int rem = m - full * big_rows;
-  t.mt = sched_cover_mt(rem, p.big_mt);
-  t.nt = sched_nt_for(t.mt, p);
-  t.m0 = full * big_rows;
-  t.n0 = (item - full_items) * t.nt * 64;
+  t.mt = sched_cover_mt(m, p.big_mt);
+  t.nt = 4;
+  t.m0 = 0;
+  t.n0 = item * 256;
   return t;
 }
 
+// Cost estimates in units of one tile row streamed through a CU: a heavy tile costs its padded rows; a light
+// item is bound by streaming its 256 weight rows (and its few token rows) from HBM at one CU's rate, which
+// takes as long as about 75 rows of a heavy tile.
+ESMOE_HD long sched_heavy_cost(int m, int n, const SchedPolicy& p) {
+  if (!sched_is_heavy(m, p)) return 0;
+  const int big = (p.force_mt ? p.force_mt : p.big_mt) * 16;
+  const int full = m / big, rem = m - full * big;
+  const int rows = full * big + (rem ? (p.force_mt ? big : sched_cover_mt(rem, p.big_mt) * 16) : 0);
+  return (long)(rows + 16 * sched_mtiles(m, p)) * sched_ntiles(n, 4);
+}
+ESMOE_HD long sched_light_cost(int m, int n, const SchedPolicy& p) {
+  return (long)sched_light_items(m, n, p) * (75 + m / 3);
+}
+// Workgroups of every 32 that start on the light items.
+ESMOE_HD int sched_light_share(long heavy_cost, long light_cost, const SchedPolicy& p) {
+  if (p.light_share >= 0) return p.light_share > 32 ? 32 : p.light_share;
+  if (heavy_cost <= 0 || light_cost <= 0) return 0;
+  const long total = heavy_cost + light_cost;
+  return (int)((32 * light_cost + total / 2) / total);
+}
+
+// Heavy ticket `ticket` of XCD `xcd` -> launch-wide block index (the caller compares it with the block total).
+ESMOE_HD int sched_ticket_block(int xcd, int ticket) { return (ticket / kBlkTiles) * kXcds + xcd; }
+
 // Workspace layout (int32 words).
-constexpr int kWsCounter = 0;   // next work item to hand out
-constexpr int kWsTotal = 1;     // number of work items
-constexpr int kWsHeader = 8;    // then item_start[E + 1] (by schedule position), then order[E]
-ESMOE_HD int ws_item_start(int) { return kWsHeader; }
-ESMOE_HD int ws_order(int num_experts) { return kWsHeader + num_experts + 1; }
-ESMOE_HD int ws_words(int num_experts) { return kWsHeader + 2 * num_experts + 1; }
+constexpr int kWsLightCounter = 0;   // next light item to hand out
+constexpr int kWsLightTotal = 1;     // number of light items
+constexpr int kWsHeavyBlocks = 2;    // number of heavy blocks
+constexpr int kWsLightShare = 3;     // workgroups of every 32 that start on the light items
+constexpr int kWsXcdCounter = 8;     // 8 words: next heavy ticket of every XCD
+constexpr int kWsHeader = 16;        // then one record of kRecWords per schedule position, E + 1 of them
+// Record of schedule position p: first heavy block, first light item, expert index, rows (clamped at 0).
+// Record E closes the prefix sums: {heavy blocks, light items, -1, 0}.
+constexpr int kRecWords = 4;
+constexpr int kRecBlock = 0, kRecItem = 1, kRecExpert = 2, kRecRows = 3;
+ESMOE_HD int ws_rec(int pos) { return kWsHeader + pos * kRecWords; }
+ESMOE_HD int ws_words(int num_experts) { return kWsHeader + (num_experts + 1) * kRecWords; }
 
 }  // namespace esmoe

@@ -167,12 +167,20 @@ int esmoe_permute_rows(const void* in, const int32_t* dst_row, long num_pairs, i
  * Host mirrors of the device-side tile schedule, for inspection and CPU tests; they touch no GPU.
  * No counterpart in the reference (its schedule lives inside CUTLASS's grouped tile scheduler).
  * esmoe_host_schedule fills `ws_host` (esmoe_gemm_workspace_bytes(E) bytes of host memory) from host
- * copies of problem_sizes exactly as the schedule kernel fills the device workspace;
- * esmoe_host_decode_item maps work item `item` to out5 = {expert, tile rows, tile cols, m0, n0}.
+ * copies of problem_sizes exactly as the schedule kernel fills the device workspace: words 1 and 2 are
+ * the number of light items and of heavy blocks.
+ * Experts with more than 64 rows are "heavy": their tiles are handed out in blocks of 8 x 4 tiles, block b
+ * to XCD b % 8, through one ticket counter per XCD; esmoe_host_decode_heavy maps ticket `ticket` of XCD `xcd`
+ * to out5 = {expert, tile rows, tile cols, m0, n0} and returns 0, or 1 if the ticket falls outside the
+ * expert's tile grid (the kernel skips it), or 2 if that XCD's queue is exhausted.
+ * The other experts are "light": one short tile per 256 columns from a launch-wide counter;
+ * esmoe_host_decode_light maps item `item` (< word 1 of the workspace) to out5.
  */
 int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int32_t* ws_host);
-int esmoe_host_decode_item(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                           int force_bm, int item, int32_t* out5);
+int esmoe_host_decode_heavy(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
+                            int force_bm, int xcd, int ticket, int32_t* out5);
+int esmoe_host_decode_light(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
+                            int force_bm, int item, int32_t* out5);
 
 /* Message describing the calling thread's most recent failure ("" if none). */
 const char* esmoe_last_error(void);

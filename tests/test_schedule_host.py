@@ -5,22 +5,39 @@ import numpy as np
 import pytest
 
 
-def _schedule(native, rows, n, force_bm=0):
+def _schedule(native, rows, n, force_bm=0, with_origin=False):
+    """Every tile the kernel would compute: all tickets of the 8 per-XCD queues, then the light items."""
     lib = native.lib
     e = len(rows)
     ps = np.array([[m, n, 512] for m in rows], dtype=np.int32)
     ws = np.zeros(lib.esmoe_gemm_workspace_bytes(e) // 4, dtype=np.int32)
-    rc = lib.esmoe_host_schedule(ps.ctypes.data_as(ctypes.c_void_p), e, n, force_bm, ws.ctypes.data_as(ctypes.c_void_p))
+    psp, wsp = ps.ctypes.data_as(ctypes.c_void_p), ws.ctypes.data_as(ctypes.c_void_p)
+    rc = lib.esmoe_host_schedule(psp, e, n, force_bm, wsp)
     assert rc == 0, native.last_error()
-    total = int(ws[1])
-    tiles = []
+    light_total, heavy_blocks = int(ws[1]), int(ws[2])
+    tiles, origin = [], []
     out = np.zeros(5, dtype=np.int32)
-    for item in range(total):
-        rc = lib.esmoe_host_decode_item(ps.ctypes.data_as(ctypes.c_void_p), ws.ctypes.data_as(ctypes.c_void_p), e, n,
-                                        force_bm, item, out.ctypes.data_as(ctypes.c_void_p))
-        assert rc == 0
+    seen_blocks = 0
+    for xcd in range(8):
+        ticket = 0
+        while True:
+            rc = lib.esmoe_host_decode_heavy(psp, wsp, e, n, force_bm, xcd, ticket, out.ctypes.data_as(ctypes.c_void_p))
+            assert rc in (0, 1, 2), native.last_error()
+            if rc == 2:
+                break
+            if rc == 0:
+                tiles.append(tuple(int(v) for v in out))
+                origin.append(("heavy", xcd, ticket // 32))
+            ticket += 1
+        assert ticket % 32 == 0  # queues end on a block boundary
+        seen_blocks += ticket // 32
+    assert seen_blocks == heavy_blocks
+    for item in range(light_total):
+        rc = lib.esmoe_host_decode_light(psp, wsp, e, n, force_bm, item, out.ctypes.data_as(ctypes.c_void_p))
+        assert rc == 0, native.last_error()
         tiles.append(tuple(int(v) for v in out))
-    return tiles
+        origin.append(("light", item))
+    return (tiles, origin) if with_origin else tiles
 
 
 @pytest.mark.parametrize("force_bm", [0, 16, 32, 64, 128, 192, 256])
@@ -59,10 +76,39 @@ def test_auto_shapes_waste_less_than_any_single_shape(esmoe):
 def test_order_is_most_rows_first(esmoe):
     from expert_specialization_moe_amd import _native
 
-    rows = [5, 900, 0, 64, 900, 7]
-    tiles = _schedule(_native, rows, 256, 0)
-    seq = []
-    for e, *_ in tiles:
-        if not seq or seq[-1] != e:
-            seq.append(e)
-    assert seq == [1, 4, 3, 5, 0]  # ties by expert index, empty experts absent
+    rows = [5, 900, 0, 64, 900, 7, 65]
+    tiles, origin = _schedule(_native, rows, 256, 0, with_origin=True)
+    # heavy experts (more than 64 rows) in block order, light ones in item order; ties by expert index, empty absent
+    heavy = sorted((o[2] * 8 + o[1], t[0]) for t, o in zip(tiles, origin) if o[0] == "heavy")
+    light = [t[0] for t, o in zip(tiles, origin) if o[0] == "light"]
+
+    def runs(seq):
+        r = []
+        for e in seq:
+            if not r or r[-1] != e:
+                r.append(e)
+        return r
+
+    assert runs([e for _, e in heavy]) == [1, 4, 6]
+    assert runs(light) == [3, 5, 0]
+
+
+def test_heavy_blocks_are_rectangles_of_one_expert_on_one_xcd(esmoe):
+    from expert_specialization_moe_amd import _native
+
+    rows = [3841, 965, 323, 215, 70, 12]
+    n = 4096
+    tiles, origin = _schedule(_native, rows, n, 0, with_origin=True)
+    blocks = {}
+    for t, o in zip(tiles, origin):
+        if o[0] == "heavy":
+            blocks.setdefault((o[1], o[2]), []).append(t)
+    assert blocks
+    for (xcd, rnd), ts in blocks.items():
+        assert len({t[0] for t in ts}) == 1 and len(ts) <= 32
+        bm, bn = len({t[3] for t in ts}), len({t[4] for t in ts})
+        assert bm <= 8 and bm * bn <= 32 and len(ts) == bm * bn
+    # a block's weight panel is contiguous
+    for ts in blocks.values():
+        n0s = sorted({t[4] for t in ts})
+        assert n0s[-1] - n0s[0] == 256 * (len(n0s) - 1)
