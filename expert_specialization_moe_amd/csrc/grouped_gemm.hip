@@ -58,6 +58,9 @@ constexpr int kRingBytes = 148 * 1024;  // LDS ring of K-block stages
 constexpr int kMaxKB = 256;             // K <= 32768: per-tile table of weight block scales
 constexpr int kSaChunkBytes = 2 * 256 * 16;  // fp8-blockwise: two buffers of [256 rows][4 K blocks] activation scales
 constexpr int kLdsBytes = kRingBytes + 2 * kMaxKB * 4 + kSaChunkBytes;
+// mxfp8 keeps nothing outside the ring (its scales travel inside the stages), so its ring takes the whole
+// allocation: 158 KB hold three stages of a 128-row tile where 148 KB hold two.
+template <bool MX> constexpr int ring_bytes() { return MX ? kLdsBytes : kRingBytes; }
 
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   v8i r;
@@ -99,7 +102,7 @@ __device__ __forceinline__ void dma16x4(uint32_t lds_addr, const void* b0, uint3
 }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0) ; explicit" ::"n"(N) : "memory");
 }
 __device__ __forceinline__ void block_barrier() {
   asm volatile("" ::: "memory");
@@ -123,7 +126,7 @@ struct TileGeom {
   // 512-byte swizzled scale tiles, 2 for the weight rows then up to 2 for the token rows
   static constexpr int kScaleBytes = MX ? 2048 : 1024;
   static constexpr int kStageBytes = kABytes + kWBytes + kScaleBytes;
-  static constexpr int kNBuf = kRingBytes / kStageBytes >= 4 ? 4 : kRingBytes / kStageBytes;
+  static constexpr int kNBuf = ring_bytes<MX>() / kStageBytes >= 4 ? 4 : ring_bytes<MX>() / kStageBytes;
   static constexpr int kABlocks = BM / 8;                               // 8-row copy blocks of the token tile
   static constexpr int kACopies = kABlocks >= kWaves ? kABlocks / kWaves : 1;  // per wavefront
   static constexpr int kWCopies = kBN / 8 / kWaves;                     // 4
@@ -404,18 +407,23 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   };
 
   // ---- pipeline --------------------------------------------------------------------------
-  // prologue: NBUF-1 K blocks in flight
+  // prologue: the weight block scales of the whole tile ([2 column blocks][KB] floats behind the ring:
+  // wavefront w copies K blocks 64*(w & 3) .. +63 of column block w >> 2, lanes past KB repeat the last
+  // one), then NBUF-1 K blocks in flight.  The scale copy is asynchronous like the others and older than
+  // all of them, so the first wait below covers it and nothing here waits for a whole stage.
+  if constexpr (!MX) {
+    const int blk = wave >> 2, kb0 = (wave & 3) * 64;
+    if (kb0 < KB) {
+      int nb = (n0 >> 7) + blk;
+      if (nb * 128 >= N) nb = n0 >> 7;
+      const int kbi = kb0 + lane < KB ? kb0 + lane : KB - 1;
+      dma4(g.sb + ((long)e * (N >> 7) + nb) * KB, (uint32_t)kbi * 4, lds0 + kRingBytes + (blk * kMaxKB + kb0) * 4);
+    }
+  }
   if (sa4 && wave * 64 < G::BM) issue_sa_chunk(0);
 #pragma unroll
   for (int s = 0; s < NBUF - 1; s++) {
     if (s < KB) issue(s, s);
-  }
-  if constexpr (!MX) {
-    // weight block scales of the whole tile (2 column blocks x KB), read back after the first barrier
-    const int blk = tid >> 8, kbi = tid & 255;
-    int nb = (n0 >> 7) + blk;
-    if (nb * 128 >= N) nb = n0 >> 7;
-    if (kbi < KB) s_sb[blk * kMaxKB + kbi] = g.sb[((long)e * (N >> 7) + nb) * KB + kbi];
   }
   // copies outstanding per in-flight stage (the chunked scale copies are older than any stage that
   // may still be in flight when their data is needed, see the loop)
