@@ -180,16 +180,28 @@ def bench_quant(args, prob, es, W):
 
 
 def bench_swiglu_quant(args, prob, es, W):
-    """Fused SwiGLU + FP8 1x128 quantisation of a [rows, N] gate_up output (N = 2 * inter)."""
+    """Fused SwiGLU + quantisation of a [rows, N] gate_up output (N = 2 * inter): FP8 1x128 for the fp8-blockwise
+    workloads, MXFP8 (grouped, swizzled E8M0 scales) for the mxfp8 workload."""
     dev = "cuda:0"
+    mx = prob.kind == "mxfp8"
     total, inter = prob.total_rows, prob.n // 2
     x = torch.randn((total, 2 * inter), generator=torch.Generator().manual_seed(args.seed)).to(torch.bfloat16)
     xd = x.to(dev)
     q = torch.empty((total, inter), dtype=torch.uint8, device=dev)
-    sc = torch.empty((total, inter // 128), dtype=torch.float32, device=dev)
+    if mx:
+        bso_np, sf_rows = W.blockscale_offsets_of(prob.rows)
+        ps = torch.tensor([[m, prob.n, inter] for m in prob.rows], dtype=torch.int32, device=dev)
+        eo = torch.tensor(W.offsets_of(prob.rows), dtype=torch.int32, device=dev)
+        bso = torch.tensor(bso_np, dtype=torch.int32, device=dev)
+        sc = torch.empty((sf_rows * (inter // 32),), dtype=torch.uint8, device=dev)
+    else:
+        sc = torch.empty((total, inter // 128), dtype=torch.float32, device=dev)
 
     def step():
-        es.es_swiglu_quant_1x128(xd, q, sc)
+        if mx:
+            es.es_swiglu_mxfp8_grouped_quant(xd, ps, eo, bso, q, sc)
+        else:
+            es.es_swiglu_quant_1x128(xd, q, sc)
 
     for _ in range(args.warmup):
         step()
@@ -202,7 +214,7 @@ def bench_swiglu_quant(args, prob, es, W):
     stop.record()
     torch.cuda.synchronize()
     ms_per_step = start.elapsed_time(stop) / args.steps
-    nbytes = float(total) * inter * (4 + 1 + 4 / 128.0)
+    nbytes = float(total) * inter * (4 + 1 + (1 / 32.0 if mx else 4 / 128.0))
     t = ms_per_step * 1e-3
     roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": W.HBM_BYTES_PER_S / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
@@ -210,23 +222,28 @@ def bench_swiglu_quant(args, prob, es, W):
     roof["algorithmic_bytes"] = nbytes
     roof["roofline_us"] = nbytes / W.HBM_BYTES_PER_S * 1e6
     out = {
-        "metric": "fused SwiGLU + FP8 1x128 quantisation, algorithmic GB/s (bf16 [rows, 2I] in, e4m3 + fp32 scales out)",
+        "metric": ("fused SwiGLU + MXFP8 grouped quantisation, algorithmic GB/s (bf16 [rows, 2I] in, e4m3 + E8M0 scales out)" if mx else
+                   "fused SwiGLU + FP8 1x128 quantisation, algorithmic GB/s (bf16 [rows, 2I] in, e4m3 + fp32 scales out)"),
         "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 -> fp32 -> bf16 -> fp8_e4m3 + fp32 scales", "data": "synthetic",
+        "dtype": "bf16 -> fp32 -> bf16 -> fp8_e4m3 + " + ("e8m0 scales" if mx else "fp32 scales"), "data": "synthetic",
         "config": {"workload": f"{prob.name} swiglu_quant: rows={total} inter={inter} seed={args.seed}"},
         "roofline": roof,
     }
     if not args.no_cpu_baseline:
         import numpy as np
         from oracle import fp8_blockwise as ofp8
+        from oracle import mxfp8 as omx
 
         xs = x[: min(total, 256)].float().numpy()
         used, nrows = 0.0, 0
         while used < args.cpu_seconds:
             t0 = time.perf_counter()
             with np.errstate(over="ignore"):
-                ofp8.quant_act_1x128(ofp8.swiglu(xs))
+                if mx:
+                    omx.quant_rows(ofp8.swiglu(xs))
+                else:
+                    ofp8.quant_act_1x128(ofp8.swiglu(xs))
             used += time.perf_counter() - t0
             nrows += xs.shape[0]
         out["cpu_baseline"] = {"value": nbytes / total * nrows / used / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
@@ -295,17 +312,23 @@ def bench_route(args, prob, es, W):
 
 
 def bench_quant_weight(args, prob, es, W):
-    """FP8 128x128 quantisation of the workload's bf16 weights [E, N, K] (offline operand preparation)."""
+    """Quantisation of the workload's bf16 weights [E, N, K] (offline operand preparation): FP8 128x128 blocks
+    for the fp8-blockwise workloads, MXFP8 with swizzled E8M0 scales for the mxfp8 workload."""
     dev = "cuda:0"
+    mx = prob.kind == "mxfp8"
     e, n, k = prob.num_experts, prob.n, prob.k
     gen = torch.Generator().manual_seed(args.seed)
     w1 = (torch.randn((n, k), generator=gen) * 0.02).to(torch.bfloat16)
     w = w1.to(dev).unsqueeze(0).repeat(e, 1, 1).contiguous()     # same values in every expert: timing does not depend on them
     q = torch.empty((e, n, k), dtype=torch.uint8, device=dev)
-    sc = torch.empty((e, n // 128, k // 128), dtype=torch.float32, device=dev)
+    sc = (torch.empty((e, n, k // 32), dtype=torch.uint8, device=dev) if mx else
+          torch.empty((e, n // 128, k // 128), dtype=torch.float32, device=dev))
 
     def step():
-        es.es_fp8_quant_weight_128x128(w, q, sc)
+        if mx:
+            es.es_mxfp8_quant_weight(w, q, sc)
+        else:
+            es.es_fp8_quant_weight_128x128(w, q, sc)
 
     for _ in range(args.warmup):
         step()
@@ -318,7 +341,7 @@ def bench_quant_weight(args, prob, es, W):
     stop.record()
     torch.cuda.synchronize()
     ms_per_step = start.elapsed_time(stop) / args.steps
-    nbytes = float(e) * n * k * 3 + float(e) * (n // 128) * (k // 128) * 4
+    nbytes = float(e) * n * k * 3 + (float(e) * n * (k // 32) if mx else float(e) * (n // 128) * (k // 128) * 4)
     t = ms_per_step * 1e-3
     roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": W.HBM_BYTES_PER_S / 1e9, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
@@ -326,10 +349,11 @@ def bench_quant_weight(args, prob, es, W):
     roof["algorithmic_bytes"] = nbytes
     roof["roofline_us"] = nbytes / W.HBM_BYTES_PER_S * 1e6
     out = {
-        "metric": "FP8 128x128 weight quantisation, algorithmic GB/s (bf16 in, e4m3 + fp32 scales out)",
+        "metric": ("MXFP8 weight quantisation, algorithmic GB/s (bf16 in, e4m3 + E8M0 scales out)" if mx else
+                   "FP8 128x128 weight quantisation, algorithmic GB/s (bf16 in, e4m3 + fp32 scales out)"),
         "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 -> fp8_e4m3 + fp32 scales", "data": "synthetic",
+        "dtype": "bf16 -> fp8_e4m3 + " + ("e8m0 scales" if mx else "fp32 scales"), "data": "synthetic",
         "config": {"workload": f"{prob.name} quant_weight: E={e} N={n} K={k} seed={args.seed}"},
         "roofline": roof,
     }
@@ -337,12 +361,16 @@ def bench_quant_weight(args, prob, es, W):
         calibration_copy()
     if not args.no_cpu_baseline:
         from oracle import fp8_blockwise as ofp8
+        from oracle import mxfp8 as omx
 
         ws = w1[: min(n, 512)].float().numpy()
         used, nrows = 0.0, 0
         while used < args.cpu_seconds:
             t0 = time.perf_counter()
-            ofp8.quant_weight_128x128(ws)
+            if mx:
+                omx.quant_rows(ws)
+            else:
+                ofp8.quant_weight_128x128(ws)
             used += time.perf_counter() - t0
             nrows += ws.shape[0]
         out["cpu_baseline"] = {"value": nrows * k * 3.0 / used / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",

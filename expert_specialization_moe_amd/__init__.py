@@ -17,6 +17,8 @@ from .ops import (  # noqa: F401
     es_route_metadata,
     es_permute_rows,
     es_swiglu_quant_1x128,
+    es_swiglu_mxfp8_grouped_quant,
+    es_mxfp8_quant_weight,
 )
 
 __all__ = [
@@ -28,4 +30,6 @@ __all__ = [
     "es_route_metadata",
     "es_permute_rows",
     "es_swiglu_quant_1x128",
+    "es_swiglu_mxfp8_grouped_quant",
+    "es_mxfp8_quant_weight",
 ]

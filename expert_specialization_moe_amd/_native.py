@@ -40,6 +40,10 @@ lib.esmoe_mxfp8_grouped_mm.restype = _i
 lib.esmoe_mxfp8_grouped_mm.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]
 lib.esmoe_mxfp8_grouped_quant.restype = _i
 lib.esmoe_mxfp8_grouped_quant.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
+lib.esmoe_swiglu_mxfp8_grouped_quant.restype = _i
+lib.esmoe_swiglu_mxfp8_grouped_quant.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
+lib.esmoe_mxfp8_quant_weight.restype = _i
+lib.esmoe_mxfp8_quant_weight.argtypes = [_vp, _i, _vp, _vp, ctypes.c_long, _i, _vp]
 lib.esmoe_fp8_quant_act_1x128.restype = _i
 lib.esmoe_fp8_quant_act_1x128.argtypes = [_vp, _i, _vp, _vp, ctypes.c_long, _i, _vp]
 lib.esmoe_fp8_quant_weight_128x128.restype = _i

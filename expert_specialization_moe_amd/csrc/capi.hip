@@ -16,7 +16,8 @@
 extern "C" int esmoe_launch_grouped_gemm(const esmoe::GemmArgs* args, int mx, int grid, hipStream_t stream);
 extern "C" int esmoe_launch_mxfp8_quant(const void* in, int in_dtype, const int* problem_sizes,
                                         const int* expert_offsets, const int* blockscale_offsets, void* q, uint8_t* sf,
-                                        int num_experts, int sf_rows, int k, hipStream_t stream);
+                                        int num_experts, long sf_rows, int k, int swiglu, long dense_rows,
+                                        hipStream_t stream);
 
 extern "C" int esmoe_launch_fp8_quant_act(const void* in, int in_dtype, void* q, float* scales, long total_rows, int k,
                                           hipStream_t stream);
@@ -176,9 +177,10 @@ int esmoe_mxfp8_grouped_mm(void* d, int out_dtype, const void* a, const void* b,
   return launch_gemm(g, 1, force_bm, stream);
 }
 
-int esmoe_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* problem_sizes,
-                              const int32_t* expert_offsets, const int32_t* blockscale_offsets, void* q,
-                              uint8_t* sf, int num_experts, int total_rows, int sf_rows, int k, void* stream) {
+namespace {
+int grouped_quant_common(const void* in, int in_dtype, const int32_t* problem_sizes, const int32_t* expert_offsets,
+                         const int32_t* blockscale_offsets, void* q, uint8_t* sf, int num_experts, int total_rows,
+                         int sf_rows, int k, int swiglu, void* stream) {
   g_err[0] = 0;
   if (!in || !problem_sizes || !expert_offsets || !blockscale_offsets || !q || !sf)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
@@ -196,7 +198,42 @@ int esmoe_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* probl
   int rc = current_device_info(&info);
   if (rc) return rc;
   rc = esmoe_launch_mxfp8_quant(in, in_dtype, problem_sizes, expert_offsets, blockscale_offsets, q, sf, num_experts,
-                                sf_rows, k, (hipStream_t)stream);
+                                sf_rows, k, swiglu, 0, (hipStream_t)stream);
+  if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return 0;
+}
+}  // namespace
+
+int esmoe_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* problem_sizes,
+                              const int32_t* expert_offsets, const int32_t* blockscale_offsets, void* q,
+                              uint8_t* sf, int num_experts, int total_rows, int sf_rows, int k, void* stream) {
+  return grouped_quant_common(in, in_dtype, problem_sizes, expert_offsets, blockscale_offsets, q, sf, num_experts,
+                              total_rows, sf_rows, k, 0, stream);
+}
+
+int esmoe_swiglu_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* problem_sizes,
+                                     const int32_t* expert_offsets, const int32_t* blockscale_offsets, void* q,
+                                     uint8_t* sf, int num_experts, int total_rows, int sf_rows, int inter,
+                                     void* stream) {
+  return grouped_quant_common(in, in_dtype, problem_sizes, expert_offsets, blockscale_offsets, q, sf, num_experts,
+                              total_rows, sf_rows, inter, 1, stream);
+}
+
+int esmoe_mxfp8_quant_weight(const void* in, int in_dtype, void* q, uint8_t* sf, long rows, int k, void* stream) {
+  g_err[0] = 0;
+  if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must align to 128, got %d", k);
+  if (in_dtype != ESMOE_IN_BF16 && in_dtype != ESMOE_IN_FP16)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in_dtype must be ESMOE_IN_BF16 or ESMOE_IN_FP16");
+  if (rows < 0 || rows % 128 || rows > (1L << 31) - 128)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "rows must be a non-negative multiple of 128 below 2^31, got %ld", rows);
+  if (rows == 0) return 0;
+  if (!in || !q || !sf) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if ((uintptr_t)in % 16 || (uintptr_t)q % 8 || (uintptr_t)sf % 16)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "in and sf must be 16-byte aligned, q 8-byte aligned");
+  DeviceInfo info;
+  int rc = current_device_info(&info);
+  if (rc) return rc;
+  rc = esmoe_launch_mxfp8_quant(in, in_dtype, nullptr, nullptr, nullptr, q, sf, 1, rows, k, 0, rows, (hipStream_t)stream);
   if (rc) return fail(rc, "quant launch failed: %s", hipGetErrorString((hipError_t)rc));
   return 0;
 }

@@ -615,7 +615,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   int phase = 0, q = 0;
 #ifdef ESMOE_TIMELINE
   int tl_n = 0;
-  if (threadIdx.x == 0) ((uint32_t*)ws)[4096 + blockIdx.x * 128] = 0;
+  if (threadIdx.x == 0) ((uint32_t*)ws)[4096 + blockIdx.x * 256] = 0;
 #endif
   for (;;) {
     const bool light = (phase == 0) == light_first;
@@ -665,14 +665,14 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
       default: break;
     }
 #ifdef ESMOE_TIMELINE
-    // debug build only: (start, end, kind) of this workgroup's first 31 tiles, in 100 MHz ticks, into a
-    // caller-provided oversize workspace from word 4096 on
+    // debug build only: (start, end, kind, position) of this workgroup's first 31 tiles, in 100 MHz ticks, 8 words
+    // per tile, into a caller-provided oversize workspace from word 4096 on
     if (threadIdx.x == 0 && tl_n < 31) {
-      uint32_t* tl = (uint32_t*)ws + 4096 + blockIdx.x * 128;
-      tl[4 + tl_n * 4 + 0] = (uint32_t)tl_t0;
-      tl[4 + tl_n * 4 + 1] = (uint32_t)__builtin_amdgcn_s_memrealtime();
-      tl[4 + tl_n * 4 + 2] = (uint32_t)(t.mt | (light ? 256 : 0) | (xcd << 12) | (e << 16));
-      tl[4 + tl_n * 4 + 3] = (uint32_t)(t.m0 / 16) | ((uint32_t)(t.n0 / 256) << 16);
+      uint32_t* tl = (uint32_t*)ws + 4096 + blockIdx.x * 256;
+      tl[8 + tl_n * 8 + 0] = (uint32_t)tl_t0;
+      tl[8 + tl_n * 8 + 1] = (uint32_t)__builtin_amdgcn_s_memrealtime();
+      tl[8 + tl_n * 8 + 2] = (uint32_t)(t.mt | (light ? 256 : 0) | (xcd << 12) | (e << 16));
+      tl[8 + tl_n * 8 + 3] = (uint32_t)(t.m0 / 16) | ((uint32_t)(t.n0 / 256) << 16);
       tl[0] = ++tl_n;
     }
 #endif

@@ -13,6 +13,14 @@
 // segment), 4 lanes share one 32-wide block and reduce amax with two lane swaps.
 // The 512-byte scale tile (128 rows x 4 scale columns, layout ((32,4),4):((16,4),1),
 // group_quant.cuh:25) is assembled in LDS and written with 16-byte stores.
+//
+// Two more forms of the same kernel (no counterpart in the reference, which quantises weights by passing
+// the activation operator a transposed problem list, test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:53,87-96,
+// and leaves the activation function to its callers):
+//   * dense: no metadata, all `dense_rows` rows (a multiple of 128) belong to one problem.  That is the
+//     weight tensor [E, N, K] with N % 128 == 0, whose scale layout is the concatenation of the experts';
+//   * SwiGLU: the input is the gate_up projection [rows, 2K]; x = silu(gate) * up with gate the first half of
+//     a row, the product formed in fp32 and rounded once to the input type, then quantised as above.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -47,38 +55,60 @@ __device__ __forceinline__ int mx_scale_code(float amax) {
 }
 
 template <bool FP16>
-__global__ void __launch_bounds__(kQuantThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) mxfp8_quant_kernel(const uint16_t* __restrict__ in,
+__device__ __forceinline__ float round_to_input_type(float h) {
+  if constexpr (FP16) return (float)(_Float16)h;
+  else return (float)(__bf16)h;
+}
+
+template <bool FP16, bool SWIGLU>
+__global__ void __launch_bounds__(kQuantThreads) __attribute__((amdgpu_waves_per_eu(SWIGLU ? 4 : 6, 8))) mxfp8_quant_kernel(const uint16_t* __restrict__ in,
                                                                     const int* __restrict__ problem_sizes,
                                                                     const int* __restrict__ expert_offsets,
                                                                     const int* __restrict__ blockscale_offsets,
                                                                     uint8_t* __restrict__ q, uint8_t* __restrict__ sf,
-                                                                    int num_experts, int k) {
+                                                                    int num_experts, int k, long dense_rows) {
   __shared__ __attribute__((aligned(16))) uint8_t s_sf[512];
   const int kt = blockIdx.x;               // 128-column tile
   const int sf_row0 = blockIdx.y * 128;    // first row of this tile in scale-row space
   const int tid = threadIdx.x;
 
-  // expert owning scale row sf_row0: last e with blockscale_offsets[e] <= sf_row0
-  int lo = 0, hi = num_experts;
-  while (hi - lo > 1) {
-    int mid = (lo + hi) >> 1;
-    if (blockscale_offsets[mid] <= sf_row0) lo = mid; else hi = mid;
+  int m_e, r0;
+  long row_base, sf_base;
+  if (dense_rows > 0) {
+    m_e = (int)dense_rows;
+    r0 = sf_row0;
+    row_base = 0;
+    sf_base = 0;
+  } else {
+    // expert owning scale row sf_row0: last e with blockscale_offsets[e] <= sf_row0
+    int lo = 0, hi = num_experts;
+    while (hi - lo > 1) {
+      int mid = (lo + hi) >> 1;
+      if (blockscale_offsets[mid] <= sf_row0) lo = mid; else hi = mid;
+    }
+    const int e = lo;
+    m_e = problem_sizes[e * 3];
+    r0 = sf_row0 - blockscale_offsets[e];  // first row of the tile inside the expert
+    row_base = expert_offsets[e];
+    sf_base = blockscale_offsets[e];
   }
-  const int e = lo;
-  const int m_e = problem_sizes[e * 3];
-  const int r0 = sf_row0 - blockscale_offsets[e];  // first row of the tile inside the expert
-  if (r0 < 0 || r0 >= m_e) return;                 // tile past the expert's rows: nothing defined there
-  const long row_base = expert_offsets[e];
+  if (r0 < 0 || r0 >= m_e) return;           // tile past the expert's rows: nothing defined there
   const int kcols = k >> 5;
+  const long in_stride = SWIGLU ? 2L * k : k;   // SwiGLU reads [rows, 2K]: gate | up
 
   const int sub = tid & 15;        // 16-byte column of the row: elements [8*sub, 8*sub + 8)
   const int rrow = tid >> 4;       // row within a 16-row pass
-  v4i raw[8];
+  v4i raw[8], rup[SWIGLU ? 8 : 1];
 #pragma unroll
   for (int p = 0; p < 8; p++) {
     int r = r0 + p * 16 + rrow;
     raw[p] = v4i{0, 0, 0, 0};
-    if (r < m_e) raw[p] = __builtin_nontemporal_load((const v4i*)(in + (row_base + r) * k + kt * 128 + sub * 8));
+    if constexpr (SWIGLU) rup[p] = v4i{0, 0, 0, 0};
+    if (r < m_e) {
+      const uint16_t* src = in + (row_base + r) * in_stride + kt * 128 + sub * 8;
+      raw[p] = __builtin_nontemporal_load((const v4i*)src);
+      if constexpr (SWIGLU) rup[p] = __builtin_nontemporal_load((const v4i*)(src + k));
+    }
   }
 #pragma unroll
   for (int p = 0; p < 8; p++) {
@@ -86,6 +116,12 @@ __global__ void __launch_bounds__(kQuantThreads) __attribute__((amdgpu_waves_per
     const int r = r0 + rt;
     float x[8];
     unpack8<FP16>(raw[p], x);
+    if constexpr (SWIGLU) {
+      float u[8];
+      unpack8<FP16>(rup[p], u);
+#pragma unroll
+      for (int i = 0; i < 8; i++) x[i] = round_to_input_type<FP16>((x[i] / (1.0f + expf(-x[i]))) * u[i]);
+    }
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) amax = __builtin_fmaxf(amax, __builtin_fabsf(x[i]));
@@ -107,24 +143,29 @@ __global__ void __launch_bounds__(kQuantThreads) __attribute__((amdgpu_waves_per
   }
   __syncthreads();
   if (tid < 32) {
-    uint8_t* dst = sf + (long)blockscale_offsets[e] * kcols + ((long)(r0 >> 7) * (k >> 7) + kt) * 512;
+    uint8_t* dst = sf + sf_base * kcols + ((long)(r0 >> 7) * (k >> 7) + kt) * 512;
     *(v4i*)(dst + tid * 16) = *(const v4i*)(s_sf + tid * 16);
   }
 }
 
 }  // namespace esmoe
 
+// swiglu != 0: `in` is [rows, 2k].  dense_rows > 0: no metadata (the three pointers may be null).
 extern "C" int esmoe_launch_mxfp8_quant(const void* in, int in_dtype, const int* problem_sizes,
                                         const int* expert_offsets, const int* blockscale_offsets, void* q, uint8_t* sf,
-                                        int num_experts, int sf_rows, int k, hipStream_t stream) {
+                                        int num_experts, long sf_rows, int k, int swiglu, long dense_rows,
+                                        hipStream_t stream) {
   using namespace esmoe;
-  dim3 grid(k / 128, sf_rows / 128);
+  dim3 grid(k / 128, (unsigned)(sf_rows / 128));
   if (grid.x == 0 || grid.y == 0) return 0;
-  if (in_dtype == 1)
-    hipLaunchKernelGGL(mxfp8_quant_kernel<true>, grid, dim3(kQuantThreads), 0, stream, (const uint16_t*)in,
-                       problem_sizes, expert_offsets, blockscale_offsets, (uint8_t*)q, sf, num_experts, k);
-  else
-    hipLaunchKernelGGL(mxfp8_quant_kernel<false>, grid, dim3(kQuantThreads), 0, stream, (const uint16_t*)in,
-                       problem_sizes, expert_offsets, blockscale_offsets, (uint8_t*)q, sf, num_experts, k);
+#define ESMOE_LAUNCH_QUANT(F16_, SW_)                                                                               \
+  hipLaunchKernelGGL((mxfp8_quant_kernel<F16_, SW_>), grid, dim3(kQuantThreads), 0, stream, (const uint16_t*)in,    \
+                     problem_sizes, expert_offsets, blockscale_offsets, (uint8_t*)q, sf, num_experts, k, dense_rows)
+  if (in_dtype == 1) {
+    if (swiglu) ESMOE_LAUNCH_QUANT(true, true); else ESMOE_LAUNCH_QUANT(true, false);
+  } else {
+    if (swiglu) ESMOE_LAUNCH_QUANT(false, true); else ESMOE_LAUNCH_QUANT(false, false);
+  }
+#undef ESMOE_LAUNCH_QUANT
   return (int)hipGetLastError();
 }

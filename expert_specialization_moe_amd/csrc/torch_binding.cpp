@@ -329,6 +329,73 @@ void es_fp8_quant_weight_128x128(const torch::Tensor& input, torch::Tensor& quan
   check_rc(rc, "es_fp8_quant_weight_128x128");
 }
 
+// Fused SwiGLU + MXFP8 grouped quantisation: the gate_up output [rows, 2*inter] -> the down projection's operands
+// (no counterpart in the reference; metadata and output layouts as es_sm100_mxfp8_blockscaled_grouped_quant with K = inter).
+void es_swiglu_mxfp8_grouped_quant(const torch::Tensor& input, const torch::Tensor& problem_sizes,
+                                   const torch::Tensor& expert_offsets, const torch::Tensor& blockscale_offsets,
+                                   torch::Tensor& quant_output, torch::Tensor& scale_factor) {
+  TORCH_CHECK(input.dim() == 2 && input.is_contiguous(), "input must be a contiguous 2D tensor");
+  TORCH_CHECK(input.size(1) % 256 == 0, "the row length must be 2 * inter with inter aligned to 128");
+  TORCH_CHECK(input.scalar_type() == torch::kBFloat16 || input.scalar_type() == torch::kHalf,
+              "dtype must be kFloat16 or kBFloat16");
+  TORCH_CHECK(problem_sizes.dim() == 2 && problem_sizes.size(1) == 3, "problem_sizes must be (groups, 3)");
+  const int64_t groups = problem_sizes.size(0);
+  TORCH_CHECK(expert_offsets.dim() == 1 && expert_offsets.size(0) == groups && blockscale_offsets.dim() == 1 &&
+                  blockscale_offsets.size(0) == groups,
+              "expert_offsets and blockscale_offsets must be 1D and have size equal to the number of groups");
+  TORCH_CHECK(problem_sizes.dtype() == torch::kInt32 && expert_offsets.dtype() == torch::kInt32 &&
+                  blockscale_offsets.dtype() == torch::kInt32,
+              "problem_sizes, expert_offsets and blockscale_offsets must be int32");
+  TORCH_CHECK(groups >= 1 && groups <= ESMOE_MAX_EXPERTS, "number of groups must be in [1, 1024]");
+  const int64_t total_rows = input.size(0), inter = input.size(1) / 2;
+  TORCH_CHECK(quant_output.is_contiguous() && (int64_t)quant_output.nbytes() >= total_rows * inter,
+              "quant_output must be contiguous and hold at least rows * inter bytes");
+  TORCH_CHECK(scale_factor.is_contiguous() && scale_factor.element_size() == 1,
+              "scale_factor must be a contiguous 1-byte tensor");
+  const int64_t sf_rows = (scale_factor.numel() / (inter / 32)) / 128 * 128;
+  TORCH_CHECK(total_rows < (int64_t(1) << 31) && sf_rows < (int64_t(1) << 31), "tensor too large");
+  require_device(input, "es_swiglu_mxfp8_grouped_quant");
+  for (const torch::Tensor* t : {&problem_sizes, &expert_offsets, &blockscale_offsets, (const torch::Tensor*)&quant_output,
+                                 (const torch::Tensor*)&scale_factor}) {
+    TORCH_CHECK(t->device() == input.device(), "all tensors must be on the same device");
+  }
+  TORCH_CHECK(problem_sizes.is_contiguous() && expert_offsets.is_contiguous() && blockscale_offsets.is_contiguous(),
+              "metadata tensors must be contiguous");
+  if (total_rows == 0) return;
+  c10::DeviceGuard guard(input.device());
+  int rc = esmoe_swiglu_mxfp8_grouped_quant(
+      input.data_ptr(), input.scalar_type() == torch::kBFloat16 ? ESMOE_IN_BF16 : ESMOE_IN_FP16,
+      problem_sizes.data_ptr<int32_t>(), expert_offsets.data_ptr<int32_t>(), blockscale_offsets.data_ptr<int32_t>(),
+      quant_output.data_ptr(), (uint8_t*)scale_factor.data_ptr(), (int)groups, (int)total_rows, (int)sf_rows, (int)inter,
+      current_stream(input));
+  check_rc(rc, "es_swiglu_mxfp8_grouped_quant");
+}
+
+// MXFP8 quantisation of a weight tensor [..., N, K] (no counterpart among the reference's operators: its test
+// passes the activation operator a transposed problem list, test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:87-96).
+void es_mxfp8_quant_weight(const torch::Tensor& input, torch::Tensor& quant_output, torch::Tensor& scale_factor) {
+  TORCH_CHECK(input.dim() >= 2, "input must have at least 2 dimensions");
+  const int64_t k = input.size(-1), n = input.size(-2);
+  TORCH_CHECK(k % 128 == 0 && n % 128 == 0, "n and k must align to 128");
+  TORCH_CHECK(input.scalar_type() == torch::kBFloat16 || input.scalar_type() == torch::kHalf,
+              "dtype must be kFloat16 or kBFloat16");
+  TORCH_CHECK(input.is_contiguous(), "input must be contiguous");
+  const int64_t rows = input.numel() / k;
+  TORCH_CHECK(quant_output.is_contiguous() && quant_output.element_size() == 1 && quant_output.numel() == rows * k,
+              "quant_output must be a contiguous 1-byte tensor with the input's number of elements");
+  TORCH_CHECK(scale_factor.is_contiguous() && scale_factor.element_size() == 1 && scale_factor.numel() == rows * (k / 32),
+              "scale_factor must be a contiguous 1-byte tensor of rows * k / 32 elements");
+  require_device(input, "es_mxfp8_quant_weight");
+  TORCH_CHECK(quant_output.device() == input.device() && scale_factor.device() == input.device(),
+              "all tensors must be on the same device");
+  if (rows == 0) return;
+  c10::DeviceGuard guard(input.device());
+  int rc = esmoe_mxfp8_quant_weight(input.data_ptr(), input.scalar_type() == torch::kBFloat16 ? ESMOE_IN_BF16 : ESMOE_IN_FP16,
+                                    quant_output.data_ptr(), (uint8_t*)scale_factor.data_ptr(), (long)rows, (int)k,
+                                    current_stream(input));
+  check_rc(rc, "es_mxfp8_quant_weight");
+}
+
 TORCH_LIBRARY(expert_specialization, m) {
   m.def(
       "es_fp8_blockwise_scaled_grouped_mm(Tensor output, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, Tensor "
@@ -343,6 +410,10 @@ TORCH_LIBRARY(expert_specialization, m) {
   m.def("es_fp8_quant_act_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def("es_fp8_quant_weight_128x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def("es_swiglu_quant_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
+  m.def(
+      "es_swiglu_mxfp8_grouped_quant(Tensor input, Tensor problem_sizes, Tensor expert_offsets, Tensor "
+      "blockscale_offsets, Tensor quant_output, Tensor scale_factor) -> ()");
+  m.def("es_mxfp8_quant_weight(Tensor input, Tensor quant_output, Tensor scale_factor) -> ()");
   m.def("es_route_metadata(Tensor topk_ids, int first_expert, int num_experts, int n, int k) -> (Tensor, Tensor, Tensor, Tensor)");
   m.def("es_permute_rows(Tensor input, Tensor dst_row, int topk, Tensor output) -> ()");
 }
@@ -354,6 +425,8 @@ TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
   m.impl("es_swiglu_quant_1x128", &es_swiglu_quant_1x128);
+  m.impl("es_swiglu_mxfp8_grouped_quant", &es_swiglu_mxfp8_grouped_quant);
+  m.impl("es_mxfp8_quant_weight", &es_mxfp8_quant_weight);
   m.impl("es_route_metadata", &es_route_metadata);
   m.impl("es_permute_rows", &es_permute_rows);
 }
@@ -366,6 +439,8 @@ TORCH_LIBRARY_IMPL(expert_specialization, CPU, m) {
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
   m.impl("es_swiglu_quant_1x128", &es_swiglu_quant_1x128);
+  m.impl("es_swiglu_mxfp8_grouped_quant", &es_swiglu_mxfp8_grouped_quant);
+  m.impl("es_mxfp8_quant_weight", &es_mxfp8_quant_weight);
   m.impl("es_route_metadata", &es_route_metadata);
   m.impl("es_permute_rows", &es_permute_rows);
 }

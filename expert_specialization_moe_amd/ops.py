@@ -86,3 +86,24 @@ def es_swiglu_quant_1x128(input, quant_output=None, scales=None):
         scales = torch.empty((m, inter // 128), dtype=torch.float32, device=input.device)
     _ns.es_swiglu_quant_1x128.default(input, quant_output, scales)
     return quant_output, scales
+
+
+def es_swiglu_mxfp8_grouped_quant(input, problem_sizes, expert_offsets, blockscale_offsets, quant_output, scale_factor):
+    """bf16/fp16 gate_up output [M, 2*I] -> MXFP8 operands of the down projection (e4m3 [M, I] + swizzled E8M0
+    scales) of silu(gate) * up in one pass; metadata and layouts as es_sm100_mxfp8_blockscaled_grouped_quant with
+    K = I (no counterpart in the reference)."""
+    _ns.es_swiglu_mxfp8_grouped_quant.default(input, problem_sizes, expert_offsets, blockscale_offsets, quant_output,
+                                              scale_factor)
+
+
+def es_mxfp8_quant_weight(input, quant_output=None, scale_factor=None):
+    """bf16/fp16 weights [..., N, K] -> (e4m3fn [..., N, K], uint8 swizzled E8M0 scales [..., N, K/32]) in the
+    layout es_sm100_mxfp8_blockscaled_grouped_mm reads as ``sfb``.  Same bytes as the reference's way of
+    quantising weights (the activation operator with the transposed problem list [N, M, K] and offsets e*N,
+    test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:53,87-96), without the metadata tensors."""
+    if quant_output is None:
+        quant_output = torch.empty(input.shape, dtype=torch.float8_e4m3fn, device=input.device)
+    if scale_factor is None:
+        scale_factor = torch.empty((*input.shape[:-1], input.shape[-1] // 32), dtype=torch.uint8, device=input.device)
+    _ns.es_mxfp8_quant_weight.default(input, quant_output, scale_factor)
+    return quant_output, scale_factor

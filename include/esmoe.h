@@ -99,6 +99,27 @@ int esmoe_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* probl
                               uint8_t* sf, int num_experts, int total_rows, int sf_rows, int k, void* stream);
 
 /*
+ * MXFP8 quantisation of a weight tensor [E, N, K] (N % 128 == 0), passed as rows = E*N rows of K: e4m3 bytes and the
+ * swizzled E8M0 scales in the layout esmoe_mxfp8_grouped_mm reads as `sfb` (expert e at byte e*N*(K/32)).  The
+ * reference has no weight entry point: its test passes the activation operator a transposed problem list
+ * [N, M, K] with offsets e*N (test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:53,87-96); this call produces
+ * the same bytes without the metadata.
+ */
+int esmoe_mxfp8_quant_weight(const void* in, int in_dtype, void* q, uint8_t* sf, long rows, int k, void* stream);
+
+/*
+ * Fused SwiGLU + MXFP8 grouped quantisation between the gate_up and the down projection: `in` is the gate_up
+ * output [total_rows, 2*inter]; x = silu(gate) * up (gate = first half of a row), formed in fp32 and rounded once
+ * to the input type, is quantised exactly as esmoe_mxfp8_grouped_quant quantises a [total_rows, inter] tensor
+ * (same q / sf layouts, same metadata, K = inter).  No counterpart in the reference, whose callers run the
+ * activation and the quantisation as separate steps.
+ */
+int esmoe_swiglu_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t* problem_sizes,
+                                     const int32_t* expert_offsets, const int32_t* blockscale_offsets, void* q,
+                                     uint8_t* sf, int num_experts, int total_rows, int sf_rows, int inter,
+                                     void* stream);
+
+/*
  * FP8 1x128 activation quantisation: bf16/fp16 rows -> e4m3fn bytes + fp32 scale per 128-wide block,
  * the `a` / `scales_a` operands of esmoe_fp8_blockwise_grouped_mm.
  * The reference has no operator for this step: its callers run the torch helper per_token_cast_to_fp8

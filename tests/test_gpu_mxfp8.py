@@ -86,3 +86,93 @@ def test_mx_end_to_end_through_ops(esmoe):
     for e, (m, off) in enumerate(zip(prob.rows, W.offsets_of(prob.rows))):
         ref = a[off:off + m] @ w[e].T
         assert calc_diff(y[off:off + m], ref) < 1e-3
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16])
+def test_weight_quant_equals_transposed_problem_list(esmoe, in_dtype):
+    """esmoe_mxfp8_quant_weight through the C ABI: bit-exact against the oracle applied the way the reference
+    quantises weights (activation operator, problem list [N, M, K], offsets e*N), and equal to this library's
+    grouped operator called that way."""
+    from expert_specialization_moe_amd import _native
+
+    e, n, k = 3, 256, 384
+    gen = torch.Generator().manual_seed(11)
+    w = (torch.randn((e, n, k), generator=gen) * 0.05).to(in_dtype)
+    w[1, 5, 32:64] = 0
+    wd = w.cuda()
+    q = torch.full((e, n, k), 0x55, dtype=torch.uint8, device="cuda")
+    sf = torch.full((e, n, k // 32), 0xEE, dtype=torch.uint8, device="cuda")
+    rc = _native.lib.esmoe_mxfp8_quant_weight(H.ptr(wd), 0 if in_dtype == torch.bfloat16 else 1, H.ptr(q), H.ptr(sf), e * n, k,
+                                              H.stream_ptr())
+    assert rc == 0, _native.last_error()
+    torch.cuda.synchronize()
+    aux_ps = [[n, 5, k]] * e
+    aux_off = [i * n for i in range(e)]
+    q_ref, sf_ref, mask = omx.grouped_quant(H.hp_to_f32(w.reshape(e * n, k)), aux_ps, aux_off, aux_off, sf_total_rows=e * n)
+    assert mask.all()
+    assert np.array_equal(q.cpu().numpy().reshape(e * n, k), q_ref)
+    assert np.array_equal(sf.cpu().numpy().reshape(-1), sf_ref)
+    # the grouped operator with the transposed problem list gives the same bytes
+    q2 = torch.zeros((e * n, k), dtype=torch.uint8, device="cuda")
+    sf2 = torch.zeros((e * n * (k // 32),), dtype=torch.uint8, device="cuda")
+    ps_d = torch.tensor(aux_ps, dtype=torch.int32, device="cuda")
+    off_d = torch.tensor(aux_off, dtype=torch.int32, device="cuda")
+    esmoe.es_sm100_mxfp8_blockscaled_grouped_quant(wd.reshape(e * n, k), ps_d, off_d, off_d, q2, sf2)
+    assert torch.equal(q2, q.reshape(e * n, k)) and torch.equal(sf2, sf.reshape(-1))
+    # operator form
+    q3, sf3 = esmoe.es_mxfp8_quant_weight(wd)
+    assert torch.equal(q3.view(torch.uint8), q) and torch.equal(sf3, sf)
+    # rows that are not a multiple of 128 are refused
+    assert _native.lib.esmoe_mxfp8_quant_weight(H.ptr(wd), 0, H.ptr(q), H.ptr(sf), 100, k, H.stream_ptr()) != 0
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16])
+def test_swiglu_mxfp8_grouped_quant_against_oracle(esmoe, in_dtype):
+    """Fused SwiGLU + MXFP8 grouped quantisation through the C ABI against oracle swiglu() -> grouped_quant().
+
+    Floating point with a transcendental (the device's fp32 exp is within an ulp or two of the oracle's correctly
+    rounded one): a product within that distance of a rounding boundary of the input type may round the other way
+    and move one quantised byte, or a block's scale when it is the block maximum at a power-of-two boundary.
+    Tolerance: at most 1e-3 of the bytes and of the scale bytes differ; zero products may carry either sign."""
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import workloads as W
+    from oracle import fp8_blockwise as ofp8
+
+    rows, inter = [3, 130, 0, 257, 64], 384
+    total = sum(rows)
+    gen = torch.Generator().manual_seed(21)
+    x = (torch.randn((total, 2 * inter), generator=gen) * 2.0).to(in_dtype)
+    x[0, :8] = torch.tensor([-100.0, -20.0, 0.0, 20.0, 100.0, -0.0, 1e-3, -1e-3]).to(in_dtype)
+    xd = x.cuda()
+    ps = [[m, 9, inter] for m in rows]
+    eo = W.offsets_of(rows)
+    bso_np, sf_rows = W.blockscale_offsets_of(rows)
+    ps_d = torch.tensor(ps, dtype=torch.int32, device="cuda")
+    eo_d = torch.tensor(eo, dtype=torch.int32, device="cuda")
+    bso_d = torch.tensor(bso_np, dtype=torch.int32, device="cuda")
+    q = torch.full((total, inter), 0x55, dtype=torch.uint8, device="cuda")
+    sf = torch.full((sf_rows * (inter // 32),), 0xEE, dtype=torch.uint8, device="cuda")
+    rc = _native.lib.esmoe_swiglu_mxfp8_grouped_quant(H.ptr(xd), 0 if in_dtype == torch.bfloat16 else 1, H.ptr(ps_d), H.ptr(eo_d),
+                                                      H.ptr(bso_d), H.ptr(q), H.ptr(sf), len(rows), total, sf_rows, inter,
+                                                      H.stream_ptr())
+    assert rc == 0, _native.last_error()
+    torch.cuda.synchronize()
+    with np.errstate(over="ignore"):
+        h = ofp8.swiglu(H.hp_to_f32(x), "bf16" if in_dtype == torch.bfloat16 else "fp16")
+    q_ref, sf_ref, mask = omx.grouped_quant(h, ps, eo, bso_np, sf_total_rows=sf_rows)
+    canon = lambda c: np.where(c == 0x80, 0, c)
+    qg, sg = q.cpu().numpy(), sf.cpu().numpy()
+    assert (canon(qg) != canon(q_ref)).mean() <= 1e-3, f"{(canon(qg) != canon(q_ref)).sum()} of {qg.size} bytes differ"
+    assert (sg[mask] != sf_ref[mask]).mean() <= 1e-3, f"{(sg[mask] != sf_ref[mask]).sum()} of {mask.sum()} scale bytes differ"
+    # the unfused sequence of this library (torch SwiGLU rounded to the input type, then the grouped quant) agrees
+    hd = (torch.nn.functional.silu(xd[:, :inter].float()) * xd[:, inter:].float()).to(in_dtype)
+    q_u = torch.zeros((total, inter), dtype=torch.uint8, device="cuda")
+    sf_u = torch.zeros_like(sf)
+    esmoe.es_sm100_mxfp8_blockscaled_grouped_quant(hd, ps_d, eo_d, bso_d, q_u, sf_u)
+    assert (canon(q_u.cpu().numpy()) != canon(qg)).mean() <= 2e-2
+    # operator form gives the bytes of the C ABI call
+    q_o = torch.zeros_like(q)
+    sf_o = torch.zeros_like(sf)
+    esmoe.es_swiglu_mxfp8_grouped_quant(xd, ps_d, eo_d, bso_d, q_o, sf_o)
+    assert torch.equal(q_o, q)
+    assert np.array_equal(sf_o.cpu().numpy()[mask], sg[mask])
