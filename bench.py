@@ -20,8 +20,8 @@ import torch
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "gemm"): 1.634e9,     # FETCH 771,376.7 x 2.000 KiB + WRITE 53,101.0 x 1.000 KiB
-    ("c4", "quant"): 1.786e8,    # FETCH 57,398.5 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
+    ("c1", "gemm"): 1.386e9,     # FETCH 650,196.3 x 2.000 KiB + WRITE 52,815.2 x 1.000 KiB
+    ("c4", "quant"): 1.786e8,    # FETCH 57,399.6 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
 }
 
 
@@ -469,6 +469,7 @@ def main():
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((prob.name, "gemm")) if not args.force_bm else None
     roof["algorithmic_bytes"] = nbytes
     roof["roofline_us"] = t_roof * 1e6
+    roof["per_expert_roofline_us"] = W.gemm_roofline_per_expert_seconds(prob.rows, n, k, prob.kind) * 1e6
     out = {
         "metric": "useful FP8 TFLOP/s + % of roofline, DSv3-shape grouped GEMM, Zipf routing",
         "value": flops / t / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

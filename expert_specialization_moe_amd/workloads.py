@@ -107,6 +107,11 @@ def gemm_roofline_seconds(rows, n, k, kind="fp8_blockwise"):
     return max(gemm_flops(rows, n, k) / FP8_FLOPS_PER_S, gemm_bytes(rows, n, k, kind) / HBM_BYTES_PER_S)
 
 
+def gemm_roofline_per_expert_seconds(rows, n, k, kind="fp8_blockwise"):
+    """Looser secondary figure: every expert priced on its own bound, sum over experts of max(F_e / P, B_e / BW)."""
+    return sum(gemm_roofline_seconds([m], n, k, kind) for m in rows if m > 0)
+
+
 # ---------------------------------------------------------------------------- operands
 def offsets_of(rows):
     off = np.zeros(len(rows), dtype=np.int64)
