@@ -49,6 +49,9 @@ def parse():
                          "route: top-k ids -> per-expert metadata + row packing of the workload's routing; "
                          "swiglu_quant: fused SwiGLU + 1x128 quantisation of the workload's [rows, N] output")
     ap.add_argument("--force-bm", type=int, default=0, help="single M-tile shape for every expert (0 = device schedule)")
+    ap.add_argument("--fuse-swiglu", action="store_true",
+                    help="gemm op, fp8-blockwise configs: the projection with the fused SwiGLU + 1x128 quantisation epilogue "
+                         "(the workload's N is read as 2 * inter); the output bytes counted are the e4m3 + scale bytes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="after the timed region also run three 1 GiB device copies (a kernel of known traffic, for "
@@ -416,7 +419,15 @@ def main():
     def vp(t):
         return ctypes.c_void_p(t.data_ptr())
 
-    if args.force_bm:
+    if args.fuse_swiglu:
+        assert not mx and n % 256 == 0, "--fuse-swiglu needs an fp8-blockwise config with N a multiple of 256"
+        q_f = torch.empty((total, n // 2), dtype=torch.uint8, device=dev)
+        sc_f = torch.empty((total, n // 256), dtype=torch.float32, device=dev)
+
+        def step():
+            es.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(q_f, sc_f, ops["a"], ops["b"], ops["scales_a"], ops["scales_b"],
+                                                               ops["problem_sizes"], ops["expert_offsets"], ops["workspace"])
+    elif args.force_bm:
         # single-tile-shape baseline: same kernel, one M-tile height for every expert (C ABI only)
         def step():
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -459,6 +470,9 @@ def main():
     flops = W.gemm_flops(prob.rows, n, k)
     nbytes = W.gemm_bytes(prob.rows, n, k, prob.kind)
     t_roof = W.gemm_roofline_seconds(prob.rows, n, k, prob.kind)
+    if args.fuse_swiglu:
+        nbytes += total * (n / 2 + 4.0 * n / 256) - 2.0 * n * total     # e4m3 + scales written instead of bf16
+        t_roof = max(flops / W.FP8_FLOPS_PER_S, nbytes / W.HBM_BYTES_PER_S)
     t = ms_per_step * 1e-3
     hbm_bound = nbytes / W.HBM_BYTES_PER_S >= flops / W.FP8_FLOPS_PER_S
     if hbm_bound:
@@ -466,7 +480,7 @@ def main():
     else:
         roof = {"bound": "mfma", "achieved": flops / t / 1e12, "peak": W.FP8_FLOPS_PER_S / 1e12, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((prob.name, "gemm")) if not args.force_bm else None
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((prob.name, "gemm")) if not (args.force_bm or args.fuse_swiglu) else None
     roof["algorithmic_bytes"] = nbytes
     roof["roofline_us"] = t_roof * 1e6
     roof["per_expert_roofline_us"] = W.gemm_roofline_per_expert_seconds(prob.rows, n, k, prob.kind) * 1e6
@@ -477,7 +491,7 @@ def main():
         "dtype": "fp8_e4m3 (fp32 accumulate, bf16 out)", "data": "synthetic",
         "config": {"workload": f"{prob.name}: E={e} K={k} N={n} rows={total} max_rows={max(prob.rows)} "
                                f"active={sum(1 for m in prob.rows if m)} kind={prob.kind} seed={args.seed}",
-                   "force_bm": args.force_bm, "routing_meta": prob.meta},
+                   "force_bm": args.force_bm, "fuse_swiglu": bool(args.fuse_swiglu), "routing_meta": prob.meta},
         "roofline": roof, "wall_ms_per_step": wall * 1e3 / args.steps,
     }
     if args.calibration_copy:

@@ -157,6 +157,28 @@ int esmoe_fp8_blockwise_grouped_mm(void* out, int out_dtype, const void* a, cons
   return launch_gemm(g, 0, force_bm, stream);
 }
 
+int esmoe_fp8_blockwise_grouped_mm_swiglu_quant(void* q, float* scales, int mid_dtype, const void* a, const void* b,
+                                                const float* sa, const float* sb, const int32_t* problem_sizes,
+                                                const int32_t* expert_offsets, int num_experts, int total_rows, int n,
+                                                int k, int force_bm, void* workspace, size_t workspace_bytes,
+                                                void* stream) {
+  g_err[0] = 0;
+  int rc = check_common(q, a, b, problem_sizes, expert_offsets, num_experts, total_rows, n, k, force_bm, workspace,
+                        workspace_bytes, mid_dtype);
+  if (rc) return rc;
+  if (!sa || !sb || !scales) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null scale pointer");
+  if (n % 256) return fail(ESMOE_ERR_INVALID_ARGUMENT, "n = 2 * inter with inter a multiple of 128, got n = %d", n);
+  if ((uintptr_t)q % 4 || (uintptr_t)scales % 4)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "q and scales must be 4-byte aligned");
+  esmoe::GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.b = b; g.sa = sa; g.sb = sb; g.q_out = q; g.scales_out = scales;
+  g.problem_sizes = problem_sizes; g.expert_offsets = expert_offsets;
+  g.ws = (int32_t*)workspace;
+  g.num_experts = num_experts; g.total_rows = total_rows; g.n = n; g.k = k; g.out_dtype = mid_dtype;
+  return launch_gemm(g, 0, force_bm, stream);
+}
+
 int esmoe_mxfp8_grouped_mm(void* d, int out_dtype, const void* a, const void* b, const uint8_t* sfa,
                            const uint8_t* sfb, const int32_t* problem_sizes, const int32_t* expert_offsets,
                            const int32_t* blockscale_offsets, int num_experts, int total_rows, int n, int k,

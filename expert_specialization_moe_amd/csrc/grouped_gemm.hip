@@ -142,8 +142,13 @@ struct TileGeom {
   static_assert(kNBuf >= 2, "ring too small");
 };
 
-template <int MT, bool MX>
+// FUSE (fp8-blockwise only): the weights are a gate_up projection [E, 2I, K] (gate rows first) and the tile's 256
+// weight rows are 128 gate rows and the matching 128 up rows, interleaved so that every wavefront holds gate and up
+// of the same columns; the epilogue forms silu(gate) * up and quantises the 128-wide block (one scale per row),
+// writing e4m3 bytes and fp32 scales instead of the bf16 projection.
+template <int MT, bool MX, bool FUSE>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds) {
+  static_assert(!(MX && FUSE), "the fused SwiGLU epilogue exists for fp8-blockwise only");
   using G = TileGeom<MT, MX>;
   constexpr int MTW = G::MTW, NTW = G::NTW, NBUF = G::kNBuf;
   const int tid = threadIdx.x;
@@ -171,7 +176,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   const uint32_t ro_even = (uint32_t)crow * (uint32_t)K + ((cslot ^ (crow >> 1)) << 4);
   const uint32_t ro_odd = ro_even ^ 64u;
   const uint8_t* a_base = (const uint8_t*)g.a + (row_base + m0) * K;
-  const uint8_t* w_base = (const uint8_t*)g.b + ((long)e * N + n0) * K;
+  const uint8_t* w_base = (const uint8_t*)g.b + ((long)e * N + (FUSE ? 0 : n0)) * K;
   const int a_last = M - 1 - m0;   // last valid token row of the tile
   // scales
   const uint8_t* sc_base;
@@ -217,8 +222,17 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
   for (int i = 0; i < G::kWCopies; i++) {
     const int blk = wave * G::kWCopies + i;
-    const int src = n0 + blk * 8 < N ? blk : i;
-    w_off[i] = (long)src * 8 * K - i * 1024;
+    if constexpr (FUSE) {
+      // LDS rows of wavefront column c (RW rows): RW/2 gate rows of columns n0/2 + c*RW/2 .., then the up rows
+      // of the same columns (weight rows I + ...)
+      constexpr int kRW = NTW * 16, kBlocks = kRW / 8, kHalfBlocks = kBlocks / 2;
+      const int wcol = blk / kBlocks, within = blk % kBlocks;
+      const int row = (within / kHalfBlocks) * (N >> 1) + (n0 >> 1) + wcol * (kRW / 2) + (within % kHalfBlocks) * 8;
+      w_off[i] = (long)row * K - i * 1024;
+    } else {
+      const int src = n0 + blk * 8 < N ? blk : i;
+      w_off[i] = (long)src * 8 * K - i * 1024;
+    }
   }
   auto issue_a = [&](int kb, int buf) {
     const uint32_t sb = lds0 + buf * G::kStageBytes;
@@ -268,7 +282,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   const int afrag_lo = (mw + r) * 128 + swz(r, gq) * 16;
   const int wfrag_lo = G::kABytes + (nw + r) * 128 + swz(r, gq) * 16;
   constexpr int kScaleOff = G::kABytes + G::kWBytes;
-  const float* sb_tab = s_sb + (nw >> 7) * kMaxKB;
+  const float* sb_tab = s_sb + (FUSE ? 0 : (nw >> 7)) * kMaxKB;   // FUSE: table 0 = gate block, table 1 = up block
   // mxfp8: per-lane bases of the scale dwords (weight rows nw + r, token rows mw + r of a tall tile)
   const int sfw_lane = kScaleOff + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16;
   const int sfa_lane = kScaleOff + 1024 + (mw >> 7) * 512 + ((mw & 127) >> 5) * 4 + r * 16;
@@ -294,6 +308,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     int sfa[MX ? MTW : 1];
     float sc[MX ? 1 : MTW];   // fp8-blockwise: sa of the row tiles (the product with sb is formed in the mfma phase)
     float sb;
+    float sb_up;   // FUSE: scale of the up rows' weight block (sb is the gate rows')
   };
 
   auto read_phase = [&](int kb, int buf, Frags& f) {
@@ -333,6 +348,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       }
     } else {
       f.sb = sb_tab[kb];
+      if constexpr (FUSE) f.sb_up = sb_tab[kMaxKB + kb];
 #pragma unroll
       for (int mt = 0; mt < MTW; mt++) {
         f.sc[mt] = sa4 ? *(const float*)(lds + sa4_lane + ((kb >> 2) & 1) * 4096 + (kb & 3) * 4 + mt * 256)
@@ -349,9 +365,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     const uint8_t* lb = lds + buf * G::kStageBytes;
     if constexpr (!MX && kPre == MTW) {
       // all fragments are in registers: one scheduling region in which promotion j - LAG issues behind MFMA j
-      float sc[MTW];
+      float sc[MTW], sc_up[FUSE ? MTW : 1];
 #pragma unroll
-      for (int mt = 0; mt < MTW; mt++) sc[mt] = f.sc[mt] * f.sb;
+      for (int mt = 0; mt < MTW; mt++) {
+        sc[mt] = f.sc[mt] * f.sb;
+        if constexpr (FUSE) sc_up[mt] = f.sc[mt] * f.sb_up;
+      }
       v4f t[MTW][NTW];
 #pragma unroll
       for (int mt = 0; mt < MTW; mt++)
@@ -363,7 +382,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++)
 #pragma unroll
-          for (int i = 0; i < 4; i++) acc[nt][mt][i] = __builtin_fmaf(t[mt][nt][i], sc[mt], acc[nt][mt][i]);
+          for (int i = 0; i < 4; i++)
+            acc[nt][mt][i] = __builtin_fmaf(t[mt][nt][i], (FUSE && nt >= NTW / 2) ? sc_up[FUSE ? mt : 0] : sc[mt], acc[nt][mt][i]);
       constexpr int kT = MTW * NTW, kLag = 3;
 #pragma unroll
       for (int j = 0; j < kLag; j++) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -403,7 +423,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
           for (int nt = 0; nt < NTW; nt++) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[nt][mt - 1][i] = __builtin_fmaf(tmp[(mt - 1) & 1][nt][i], f.sc[mt - 1] * f.sb, acc[nt][mt - 1][i]);
+            for (int i = 0; i < 4; i++)
+              acc[nt][mt - 1][i] = __builtin_fmaf(tmp[(mt - 1) & 1][nt][i], f.sc[mt - 1] * ((FUSE && nt >= NTW / 2) ? f.sb_up : f.sb), acc[nt][mt - 1][i]);
             asm volatile("" : "+v"(acc[nt][mt - 1]));  // keeps the promotion here, in the shadow of the MFMAs above
           }
         }
@@ -414,7 +435,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
       for (int nt = 0; nt < NTW; nt++) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[nt][MTW - 1][i] = __builtin_fmaf(tmp[(MTW - 1) & 1][nt][i], f.sc[MTW - 1] * f.sb, acc[nt][MTW - 1][i]);
+        for (int i = 0; i < 4; i++)
+          acc[nt][MTW - 1][i] = __builtin_fmaf(tmp[(MTW - 1) & 1][nt][i], f.sc[MTW - 1] * ((FUSE && nt >= NTW / 2) ? f.sb_up : f.sb), acc[nt][MTW - 1][i]);
         asm volatile("" : "+v"(acc[nt][MTW - 1]));
       }
     }
@@ -430,6 +452,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     if (kb0 < KB) {
       int nb = (n0 >> 7) + blk;
       if (nb * 128 >= N) nb = n0 >> 7;
+      if constexpr (FUSE) nb = (n0 >> 8) + blk * (N >> 8);   // gate block of these columns, up block I/128 further
       const int kbi = kb0 + lane < KB ? kb0 + lane : KB - 1;
       dma4(g.sb + ((long)e * (N >> 7) + nb) * KB, (uint32_t)kbi * 4, lds0 + kRingBytes + (blk * kMaxKB + kb0) * 4);
     }
@@ -505,6 +528,68 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   }
   if (kPP && grp == 0) block_barrier();
 
+  if constexpr (FUSE) {
+    // Lane holds, of token row mw + mt*16 + r, gate (n-tiles 0 .. NTW/2-1) and up (the other half) of the h columns
+    // wn*RW/2 + nt*16 + 4*gq + [0,4) of the tile's 128.  Same arithmetic, in the same order, as the unfused
+    // sequence: projection rounded to the output type, silu(gate) * up in fp32, rounded to the output type, then
+    // the 1x128 quantisation (block maximum floored at 1e-4, multiplier (1/amax)*448, scale amax*(1/448)).
+    constexpr int kHalf = NTW / 2, kRW = NTW * 16;
+    const bool f16 = g.out_dtype != 0;
+    float* s_amax = (float*)lds;   // [kWavesN][BM]; the ring is free: every wavefront has left the K loop
+    float h[MTW][kHalf][4];
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) {
+      float amax = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < kHalf; nt++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float gv, uv;
+          if (f16) {
+            gv = (float)(_Float16)acc[nt][mt][i];
+            uv = (float)(_Float16)acc[nt + kHalf][mt][i];
+          } else {
+            gv = (float)(__bf16)acc[nt][mt][i];
+            uv = (float)(__bf16)acc[nt + kHalf][mt][i];
+          }
+          float hv = (gv / (1.0f + expf(-gv))) * uv;
+          hv = f16 ? (float)(_Float16)hv : (float)(__bf16)hv;
+          h[mt][nt][i] = hv;
+          amax = __builtin_fmaxf(amax, __builtin_fabsf(hv));
+        }
+      }
+      amax = __builtin_fmaxf(amax, __shfl_xor(amax, 16));
+      amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32));
+      if (gq == 0) s_amax[wn * G::BM + mw + mt * 16 + r] = amax;
+    }
+    __syncthreads();
+    const int inter = N >> 1;
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) {
+      const int row = mw + mt * 16 + r;
+      float amax = 0.f;
+#pragma unroll
+      for (int w = 0; w < G::kWavesN; w++) amax = __builtin_fmaxf(amax, s_amax[w * G::BM + row]);
+      amax = __builtin_fmaxf(amax, 1e-4f);
+      const float mult = (1.0f / amax) * 448.0f;
+      const int m = m0 + row;
+      if (m < M) {
+        uint8_t* qrow = (uint8_t*)g.q_out + (row_base + m) * (long)inter + (n0 >> 1) + wn * (kRW / 2) + gq * 4;
+#pragma unroll
+        for (int nt = 0; nt < kHalf; nt++) {
+          float y[4];
+#pragma unroll
+          for (int i = 0; i < 4; i++) y[i] = __builtin_amdgcn_fmed3f(h[mt][nt][i] * mult, -448.f, 448.f);
+          int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+          w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+          *(int*)(qrow + nt * 16) = w0;
+        }
+        if (gq == 0 && wn == 0) g.scales_out[(row_base + m) * (long)(inter >> 7) + (n0 >> 8)] = amax * (1.0f / 448.0f);
+      }
+    }
+    __syncthreads();   // s_amax is ring memory: the next tile's copies must not land before every lane has read it
+    return;
+  }
   // epilogue: lane holds columns n0 + nw + nt*16 + 4*gq + [0,4) of token row m0 + mw + mt*16 + r
   if (wave_active) {
 #pragma unroll
@@ -595,7 +680,7 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 #define ESMOE_VARIANTS ESMOE_CASE(1) ESMOE_CASE(2) ESMOE_CASE(4) ESMOE_CASE(8) ESMOE_CASE(12) ESMOE_CASE(16)
 #endif
 
-template <bool MX>
+template <bool MX, bool FUSE>
 __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
   __shared__ int s_item;
@@ -604,7 +689,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   const int hblocks = ws[kWsHeavyBlocks];
   const int ltotal = ws[kWsLightTotal];
 #define ESMOE_CASE(MT_) \
-  case (MT_): gemm_tile<MT_, MX>(g, e, M, t.m0, t.n0, lds); break;
+  case (MT_): gemm_tile<MT_, MX, FUSE>(g, e, M, t.m0, t.n0, lds); break;
 
   // Workgroup i runs on XCD i % 8 (HW_REG_XCC_ID = 20, bits [3:0], says so directly).  Of every 32 workgroups
   // of an XCD the last `light_share` start on the light items, the others on the heavy tickets; either kind
@@ -689,8 +774,10 @@ extern "C" int esmoe_launch_grouped_gemm(const esmoe::GemmArgs* args, int mx, in
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return (int)err;
   if (mx)
-    hipLaunchKernelGGL(grouped_gemm_kernel<true>, dim3(grid), dim3(kThreads), 0, stream, *args);
+    hipLaunchKernelGGL((grouped_gemm_kernel<true, false>), dim3(grid), dim3(kThreads), 0, stream, *args);
+  else if (args->q_out)
+    hipLaunchKernelGGL((grouped_gemm_kernel<false, true>), dim3(grid), dim3(kThreads), 0, stream, *args);
   else
-    hipLaunchKernelGGL(grouped_gemm_kernel<false>, dim3(grid), dim3(kThreads), 0, stream, *args);
+    hipLaunchKernelGGL((grouped_gemm_kernel<false, false>), dim3(grid), dim3(kThreads), 0, stream, *args);
   return (int)hipGetLastError();
 }

@@ -110,6 +110,63 @@ void es_fp8_blockwise_scaled_grouped_mm(torch::Tensor& output, const torch::Tens
   check_rc(rc, "es_fp8_blockwise_scaled_grouped_mm");
 }
 
+// The gate_up projection with SwiGLU and 1x128 re-quantisation fused into its epilogue (no counterpart in the
+// reference).  Operand layouts as es_fp8_blockwise_scaled_grouped_mm with n = 2 * inter; `mid_dtype_bf16` selects the
+// type the projection and the activation are rounded to on the way (true: bfloat16, false: half).
+void es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(torch::Tensor& quant_output, torch::Tensor& scales_out,
+                                                     const torch::Tensor& a, const torch::Tensor& b,
+                                                     const torch::Tensor& scales_a, const torch::Tensor& scales_b,
+                                                     const torch::Tensor& problem_sizes,
+                                                     const torch::Tensor& expert_offsets, const torch::Tensor& workspace,
+                                                     bool mid_dtype_bf16) {
+  TORCH_CHECK(problem_sizes.dim() == 2 && problem_sizes.size(1) == 3, "problem_sizes must have shape (num_experts, 3)");
+  TORCH_CHECK(expert_offsets.dim() == 1 && problem_sizes.size(0) == expert_offsets.size(0),
+              "Number of experts in problem_sizes must match expert_offsets");
+  TORCH_CHECK(problem_sizes.dtype() == torch::kInt32 && expert_offsets.dtype() == torch::kInt32,
+              "problem_sizes and expert_offsets must be int32");
+  TORCH_CHECK(a.scalar_type() == torch::kFloat8_e4m3fn && b.scalar_type() == torch::kFloat8_e4m3fn,
+              "a and b must be kFloat8_e4m3fn");
+  const int64_t num_experts = problem_sizes.size(0);
+  TORCH_CHECK(num_experts >= 1 && num_experts <= ESMOE_MAX_EXPERTS, "Number of experts cannot exceed 1024");
+  TORCH_CHECK(a.dim() == 2 && a.stride(1) == 1 && a.stride(0) == a.size(1), "a must be a packed row-major (rows, k) tensor");
+  TORCH_CHECK(b.dim() == 3 && b.size(0) == num_experts, "b must be a (num_experts, k, n) tensor");
+  TORCH_CHECK(b.stride(1) == 1 && b.stride(2) == b.size(1) && b.stride(0) == b.size(1) * b.size(2),
+              "b must be the column-major (num_experts, k, n) view of a packed (num_experts, n, k) tensor");
+  const int64_t total_rows = a.size(0), k = a.size(1), n = b.size(2);
+  TORCH_CHECK(b.size(1) == k, "a and b disagree on k");
+  TORCH_CHECK(k % 128 == 0 && n % 256 == 0, "k must be a multiple of 128 and n = 2 * inter a multiple of 256");
+  const int64_t inter = n / 2;
+  TORCH_CHECK(quant_output.is_contiguous() && quant_output.element_size() == 1 && quant_output.numel() == total_rows * inter,
+              "quant_output must be a contiguous 1-byte tensor of rows * n / 2 elements");
+  TORCH_CHECK(scales_out.is_contiguous() && scales_out.scalar_type() == torch::kFloat32 &&
+                  scales_out.numel() == total_rows * (inter / 128),
+              "scales_out must be a contiguous float32 tensor of rows * n / 256 elements");
+  TORCH_CHECK(scales_a.scalar_type() == torch::kFloat32 && scales_b.scalar_type() == torch::kFloat32,
+              "scales must be float32");
+  TORCH_CHECK(scales_a.dim() == 2 && scales_a.size(0) == total_rows && scales_a.size(1) == k / 128 &&
+                  scales_a.is_contiguous(),
+              "scales_a must be a contiguous (rows, k/128) tensor");
+  TORCH_CHECK(scales_b.dim() == 3 && scales_b.size(0) == num_experts && scales_b.size(1) == k / 128 &&
+                  scales_b.size(2) == n / 128 && scales_b.stride(1) == 1 && scales_b.stride(2) == k / 128,
+              "scales_b must be the (num_experts, k/128, n/128) view of a packed (num_experts, n/128, k/128) tensor");
+  TORCH_CHECK(total_rows < (int64_t(1) << 31) && n < (int64_t(1) << 31) && k < (int64_t(1) << 31), "tensor too large");
+  require_device(a, "es_fp8_blockwise_scaled_grouped_mm_swiglu_quant");
+  for (const torch::Tensor* t : {(const torch::Tensor*)&quant_output, (const torch::Tensor*)&scales_out, &b, &scales_a,
+                                 &scales_b, &problem_sizes, &expert_offsets}) {
+    TORCH_CHECK(t->device() == a.device(), "all tensors must be on the same device");
+  }
+  TORCH_CHECK(problem_sizes.is_contiguous() && expert_offsets.is_contiguous(), "metadata tensors must be contiguous");
+  if (total_rows == 0) return;
+  c10::DeviceGuard guard(a.device());
+  torch::Tensor ws = schedule_scratch(&workspace, num_experts, a);
+  int rc = esmoe_fp8_blockwise_grouped_mm_swiglu_quant(
+      quant_output.data_ptr(), scales_out.data_ptr<float>(), mid_dtype_bf16 ? ESMOE_OUT_BF16 : ESMOE_OUT_FP16, a.data_ptr(),
+      b.data_ptr(), scales_a.data_ptr<float>(), scales_b.data_ptr<float>(), problem_sizes.data_ptr<int32_t>(),
+      expert_offsets.data_ptr<int32_t>(), (int)num_experts, (int)total_rows, (int)n, (int)k, /*force_bm=*/0, ws.data_ptr(),
+      ws.nbytes(), current_stream(a));
+  check_rc(rc, "es_fp8_blockwise_scaled_grouped_mm_swiglu_quant");
+}
+
 void es_sm100_mxfp8_blockscaled_grouped_mm(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& sfa,
                                            const torch::Tensor& sfb, torch::Tensor& d,
                                            const torch::Tensor& problem_sizes, const torch::Tensor& expert_offsets,
@@ -407,6 +464,9 @@ TORCH_LIBRARY(expert_specialization, m) {
   m.def(
       "es_sm100_mxfp8_blockscaled_grouped_quant(Tensor input, Tensor problem_sizes, Tensor expert_offsets, Tensor "
       "blockscale_offsets, Tensor quant_output, Tensor scale_factor) -> () ");
+  m.def(
+      "es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(Tensor quant_output, Tensor scales_out, Tensor a, Tensor b, Tensor "
+      "scales_a, Tensor scales_b, Tensor problem_sizes, Tensor expert_offsets, Tensor workspace, bool mid_dtype_bf16) -> ()");
   m.def("es_fp8_quant_act_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def("es_fp8_quant_weight_128x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def("es_swiglu_quant_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
@@ -422,6 +482,7 @@ TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
   m.impl("es_fp8_blockwise_scaled_grouped_mm", &es_fp8_blockwise_scaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_mm", &es_sm100_mxfp8_blockscaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
+  m.impl("es_fp8_blockwise_scaled_grouped_mm_swiglu_quant", &es_fp8_blockwise_scaled_grouped_mm_swiglu_quant);
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
   m.impl("es_swiglu_quant_1x128", &es_swiglu_quant_1x128);
@@ -436,6 +497,7 @@ TORCH_LIBRARY_IMPL(expert_specialization, CPU, m) {
   m.impl("es_fp8_blockwise_scaled_grouped_mm", &es_fp8_blockwise_scaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_mm", &es_sm100_mxfp8_blockscaled_grouped_mm);
   m.impl("es_sm100_mxfp8_blockscaled_grouped_quant", &es_sm100_mxfp8_blockscaled_grouped_quant);
+  m.impl("es_fp8_blockwise_scaled_grouped_mm_swiglu_quant", &es_fp8_blockwise_scaled_grouped_mm_swiglu_quant);
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
   m.impl("es_swiglu_quant_1x128", &es_swiglu_quant_1x128);

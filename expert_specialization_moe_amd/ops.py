@@ -107,3 +107,14 @@ def es_mxfp8_quant_weight(input, quant_output=None, scale_factor=None):
         scale_factor = torch.empty((*input.shape[:-1], input.shape[-1] // 32), dtype=torch.uint8, device=input.device)
     _ns.es_mxfp8_quant_weight.default(input, quant_output, scale_factor)
     return quant_output, scale_factor
+
+
+def es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(quant_output, scales_out, a, b, scales_a, scales_b, problem_sizes,
+                                                    expert_offsets, workspace, mid_dtype=torch.bfloat16):
+    """gate_up projection + SwiGLU + 1x128 re-quantisation in one kernel: writes the down projection's ``a``
+    (e4m3fn [M, I]) and ``scales_a`` (fp32 [M, I/128]) where ``b`` is the (E, K, 2I) view of gate_up weights
+    [E, 2I, K] (gate rows first).  Same bytes as es_fp8_blockwise_scaled_grouped_mm (output of ``mid_dtype``)
+    followed by es_swiglu_quant_1x128; no counterpart in the reference."""
+    _ns.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant.default(quant_output, scales_out, a, b, scales_a, scales_b,
+                                                                problem_sizes, expert_offsets, workspace,
+                                                                mid_dtype == torch.bfloat16)

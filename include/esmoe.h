@@ -80,6 +80,26 @@ int esmoe_mxfp8_grouped_mm(void* d, int out_dtype, const void* a, const void* b,
                            int force_bm, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * FP8-blockwise grouped GEMM of a gate_up projection with the SwiGLU and the 1x128 re-quantisation fused into its
+ * epilogue: produces the `a` / `scales_a` operands of the down projection directly, without the bf16 [total_rows, n]
+ * intermediate.  No counterpart in the reference (its callers run projection, activation and quantisation as
+ * separate steps); the arithmetic is that of esmoe_fp8_blockwise_grouped_mm followed by esmoe_swiglu_quant_1x128,
+ * step for step, so the two routes give the same bytes.
+ *
+ *   b [E, n, K] with n = 2 * inter: weight rows [0, inter) are the gate, [inter, 2 * inter) the up projection
+ *   (inter % 128 == 0); sb [E, n/128, K/128] as usual.
+ *   q [total_rows, inter] e4m3fn;  scales [total_rows, inter/128] fp32.
+ *   mid_dtype: ESMOE_OUT_BF16 / ESMOE_OUT_FP16, the type the projection and the activation are rounded to on the
+ *   way (what `out_dtype` and the activation's input type would be on the separate route).
+ * The other arguments are those of esmoe_fp8_blockwise_grouped_mm.
+ */
+int esmoe_fp8_blockwise_grouped_mm_swiglu_quant(void* q, float* scales, int mid_dtype, const void* a, const void* b,
+                                                const float* sa, const float* sb, const int32_t* problem_sizes,
+                                                const int32_t* expert_offsets, int num_experts, int total_rows, int n,
+                                                int k, int force_bm, void* workspace, size_t workspace_bytes,
+                                                void* stream);
+
+/*
  * MXFP8 grouped quantisation: bf16/fp16 rows -> e4m3 bytes + swizzled E8M0 scales.
  * Replaces es_sm100_mxfp8_blockscaled_grouped_quant
  *   (expert_specialization/csrc/cuda/es_sm100_mxfp8_blockscaled_group_quant.cu:5-39,
