@@ -216,6 +216,8 @@ int grouped_quant_common(const void* in, int in_dtype, const int32_t* problem_si
   if ((uintptr_t)in % 16 || (uintptr_t)q % 8 || (uintptr_t)sf % 16)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "in and sf must be 16-byte aligned, q 8-byte aligned");
   if (total_rows == 0 || sf_rows == 0) return 0;
+  if (sf_rows / 128 > 65535)   // one workgroup row per 128 scale rows, in the y dimension of the launch
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "sf_rows must not exceed 65535 * 128, got %d", sf_rows);
   DeviceInfo info;
   int rc = current_device_info(&info);
   if (rc) return rc;
@@ -246,8 +248,8 @@ int esmoe_mxfp8_quant_weight(const void* in, int in_dtype, void* q, uint8_t* sf,
   if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must align to 128, got %d", k);
   if (in_dtype != ESMOE_IN_BF16 && in_dtype != ESMOE_IN_FP16)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "in_dtype must be ESMOE_IN_BF16 or ESMOE_IN_FP16");
-  if (rows < 0 || rows % 128 || rows > (1L << 31) - 128)
-    return fail(ESMOE_ERR_INVALID_ARGUMENT, "rows must be a non-negative multiple of 128 below 2^31, got %ld", rows);
+  if (rows < 0 || rows % 128 || rows / 128 > 65535)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "rows must be a non-negative multiple of 128, at most 65535 * 128, got %ld", rows);
   if (rows == 0) return 0;
   if (!in || !q || !sf) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
   if ((uintptr_t)in % 16 || (uintptr_t)q % 8 || (uintptr_t)sf % 16)
