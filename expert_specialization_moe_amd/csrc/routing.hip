@@ -118,6 +118,86 @@ __global__ void __launch_bounds__(64) route_rank_kernel(const int* __restrict__ 
   }
 }
 
+// Small inputs (at most kSmallChunks chunks, at most kSmallExperts experts): the three passes in one workgroup of
+// kSmallChunks wavefronts, wavefront w owning chunk w, with the per-chunk counters in LDS instead of the workspace.
+// Same integers as the three-kernel route; saves two launches, which is most of the time at decode sizes.
+constexpr int kSmallChunks = 16;
+constexpr int kSmallExperts = 256;
+
+__global__ void __launch_bounds__(kSmallChunks * 64) route_small_kernel(const int* __restrict__ ids, long num_pairs,
+                                                                       int first_expert, int num_experts, int n, int k,
+                                                                       int* __restrict__ problem_sizes,
+                                                                       int* __restrict__ expert_offsets,
+                                                                       int* __restrict__ blockscale_offsets,
+                                                                       int* __restrict__ dst_row) {
+  __shared__ int s_cnt[kSmallChunks][kSmallExperts];   // per-chunk counts, then each chunk's next free row per expert
+  __shared__ int s_tot[kSmallExperts];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  for (int i = tid; i < kSmallChunks * kSmallExperts; i += kSmallChunks * 64) (&s_cnt[0][0])[i] = 0;
+  __syncthreads();
+  const long base = (long)w * kChunk;
+  for (int i = lane; i < kChunk; i += 64) {
+    const long p = base + i;
+    if (p < num_pairs) {
+      const int id = ids[p] - first_expert;
+      if (id >= 0 && id < num_experts) atomicAdd(&s_cnt[w][id], 1);
+    }
+  }
+  __syncthreads();
+  if (tid < num_experts) {
+    int total = 0;
+    for (int c = 0; c < kSmallChunks; c++) {
+      const int v = s_cnt[c][tid];
+      s_cnt[c][tid] = total;
+      total += v;
+    }
+    s_tot[tid] = total;
+  }
+  __syncthreads();
+  if (tid < num_experts) {
+    int off = 0, boff = 0;
+    for (int j = 0; j < tid; j++) {
+      const int c = s_tot[j];
+      off += c;
+      boff += (c + 127) & ~127;
+    }
+    const int total = s_tot[tid];
+    expert_offsets[tid] = off;
+    blockscale_offsets[tid] = boff;
+    problem_sizes[tid * 3 + 0] = total;
+    problem_sizes[tid * 3 + 1] = n;
+    problem_sizes[tid * 3 + 2] = k;
+    if (tid == num_experts - 1) {
+      expert_offsets[num_experts] = off + total;
+      blockscale_offsets[num_experts] = boff + ((total + 127) & ~127);
+    }
+    for (int c = 0; c < kSmallChunks; c++) s_cnt[c][tid] += off;
+  }
+  __syncthreads();
+  for (int step = 0; step < kChunk / 64; step++) {
+    const long p = base + step * 64 + lane;
+    if (base + step * 64 >= num_pairs) break;   // wave-uniform
+    int id = -1;
+    if (p < num_pairs) {
+      id = ids[p] - first_expert;
+      if (id < 0 || id >= num_experts) id = -1;
+    }
+    int row = -1;
+    unsigned long long todo = __ballot(id >= 0);
+    while (todo) {
+      const int leader = __builtin_ctzll(todo);
+      const int lid = __shfl(id, leader);
+      const unsigned long long same = __ballot(id == lid);
+      if (id == lid) row = s_cnt[w][lid] + __builtin_popcountll(same & ((1ull << lane) - 1ull));
+      __builtin_amdgcn_wave_barrier();
+      if (lane == leader) s_cnt[w][lid] += __builtin_popcountll(same);
+      __builtin_amdgcn_wave_barrier();
+      todo &= ~same;
+    }
+    if (p < num_pairs) dst_row[p] = row;
+  }
+}
+
 // Packs rows for the grouped operators: out[dst_row[p], :] = in[p / topk, :] for every local pair
 // (2-byte elements, row_bytes a multiple of 16).  One wavefront moves one row in 1 KB steps.
 __global__ void __launch_bounds__(256) permute_rows_kernel(const uint8_t* __restrict__ in, const int* __restrict__ dst_row,
@@ -148,6 +228,11 @@ extern "C" int esmoe_launch_route_metadata(const int* ids, long num_pairs, int f
                                            int* chunk_counts, hipStream_t stream) {
   using namespace esmoe;
   const int chunks = (int)((num_pairs + kChunk - 1) / kChunk);
+  if (chunks <= kSmallChunks && num_experts <= kSmallExperts) {
+    hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(kSmallChunks * 64), 0, stream, ids, num_pairs, first_expert,
+                       num_experts, n, k, problem_sizes, expert_offsets, blockscale_offsets, dst_row);
+    return (int)hipGetLastError();
+  }
   if (chunks > 0)
     hipLaunchKernelGGL(route_count_kernel, dim3(chunks), dim3(64), 0, stream, ids, num_pairs, first_expert, num_experts,
                        chunk_counts);

@@ -33,7 +33,8 @@ def _capi_route(native, ids, first, experts, n, k):
 @pytest.mark.parametrize("seed,pairs,experts,first,span", [(0, 0, 4, 0, 4), (1, 1, 1, 0, 1), (2, 777, 8, 16, 40), (3, 1024, 32, 0, 32),
                                                             (4, 1025, 32, 0, 256), (5, 32768, 32, 64, 256),
                                                             (6, 131072, 128, 0, 128), (7, 5000, 1024, 0, 1024),
-                                                            (8, 4096, 3, 5, 6)])
+                                                            (8, 4096, 3, 5, 6), (9, 16384, 256, 0, 300), (10, 16385, 256, 0, 300),
+                                                            (11, 6579, 32, 0, 256), (12, 16384, 257, 0, 257)])
 def test_route_metadata_bit_exact(esmoe, seed, pairs, experts, first, span):
     from expert_specialization_moe_amd import _native
 
