@@ -99,3 +99,57 @@ def test_fused_through_operator_and_untouched_rows(esmoe):
         H.ptr(ops["problem_sizes"]), H.ptr(ops["expert_offsets"]), 3, prob.total_rows, 384, 256, 0, H.ptr(ops["workspace"]),
         ops["workspace"].numel(), H.stream_ptr())
     assert rc != 0
+
+
+def test_fused_equals_separate_route_at_c1_size(esmoe):
+    """Full DeepSeek-V3 gate_up share (E=32, K=7168, N=4096, Zipf rows): the fused operator and the two separate
+    operators give identical bytes and scales; nothing outside the experts' rows is written."""
+    from expert_specialization_moe_amd import workloads as W
+
+    prob = W.config_problem("c1")
+    ops = W.make_fp8_blockwise_operands(prob, "cuda", seed=0)
+    total, inter = prob.total_rows, prob.n // 2
+    q = torch.full((total, inter), 0x55, dtype=torch.uint8, device="cuda")
+    sc = torch.full((total, inter // 128), -1.0, dtype=torch.float32, device="cuda")
+    esmoe.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(q, sc, ops["a"], ops["b"], ops["scales_a"], ops["scales_b"],
+                                                          ops["problem_sizes"], ops["expert_offsets"], ops["workspace"])
+    esmoe.es_fp8_blockwise_scaled_grouped_mm(ops["output"], ops["a"], ops["b"], ops["scales_a"], ops["scales_b"],
+                                             ops["stride_a"], ops["stride_b"], ops["stride_d"], ops["problem_sizes"],
+                                             ops["expert_offsets"], ops["workspace"])
+    q_ref, sc_ref = esmoe.es_swiglu_quant_1x128(ops["output"])
+    torch.cuda.synchronize()
+    assert torch.equal(q, q_ref.view(torch.uint8))
+    assert torch.equal(sc, sc_ref)
+    assert (sc > 0).all()
+
+
+def test_fused_replays_in_a_graph(esmoe):
+    """The fused operator captured in a HIP graph gives the eager result on every replay (no allocation, no memset
+    node: the workspace is passed in and the schedule kernel clears its own counters)."""
+    from expert_specialization_moe_amd import workloads as W
+
+    prob = W.Problem("gate_up", 512, 384, [40, 0, 300, 7])
+    ops = W.make_fp8_blockwise_operands(prob, "cuda", seed=8, weight_std=0.05)
+    total, inter = prob.total_rows, 256
+    q_e = torch.zeros((total, inter), dtype=torch.uint8, device="cuda")
+    sc_e = torch.zeros((total, inter // 128), dtype=torch.float32, device="cuda")
+    args = (ops["a"], ops["b"], ops["scales_a"], ops["scales_b"], ops["problem_sizes"], ops["expert_offsets"], ops["workspace"])
+    esmoe.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(q_e, sc_e, *args)
+    torch.cuda.synchronize()
+    q_g = torch.zeros_like(q_e)
+    sc_g = torch.zeros_like(sc_e)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        esmoe.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(q_g, sc_g, *args)   # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        esmoe.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(q_g, sc_g, *args)
+    for _ in range(3):
+        q_g.zero_()
+        sc_g.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(q_g, q_e) and torch.equal(sc_g, sc_e)
