@@ -80,34 +80,40 @@ __device__ __forceinline__ void dma16(const void* base, uint32_t voff, uint32_t 
 __device__ __forceinline__ void dma4(const void* base, uint32_t voff, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
-// Groups of copies whose LDS destinations are 1024 bytes apart share one write of m0 and use the
-// instruction's immediate offset, which the hardware adds to the LDS address and to the global
-// address alike (so base i must already have i*1024 subtracted).  Writing m0 between two copies
-// costs a wavefront on the order of 150 cycles: the write waits until the previous copy has read it.
-__device__ __forceinline__ void dma16x2(uint32_t lds_addr, const void* b0, uint32_t v0, const void* b1, uint32_t v1) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %3, %4 offset:1024"
-               ::"s"(lds_addr), "v"(v0), "s"(b0), "v"(v1), "s"(b1) : "memory", "m0");
+// Groups of copies whose LDS destinations are 1024 bytes apart share one write of m0 and one base pointer and use
+// the instruction's immediate offset, which the hardware adds to the LDS address and to the global address alike
+// (so per-lane offset i must already have i*1024 subtracted).  Writing m0 between two copies costs a wavefront on
+// the order of 150 cycles: the write waits until the previous copy has read it.  One scalar base per group keeps the
+// scalar work per K block at one 64-bit add: a wavefront issues its scalar instructions 4-5 cycles apart, and a
+// pointer per copy put 150 cycles of them between the barrier and the first copy.
+#define ESMOE_DMA1(n, nt) "global_load_lds_dwordx4 %" #n ", %1" nt
+#define ESMOE_DMAO(n, off, nt) "\n\tglobal_load_lds_dwordx4 %" #n ", %1 offset:" #off nt
+template <bool NT, int N>
+__device__ __forceinline__ void dma16xn(uint32_t lds_addr, const void* base, const uint32_t (&v)[N]) {
+  static_assert(N >= 1 && N <= 4, "copies per group");
+  if constexpr (N == 1) {
+    if constexpr (NT) asm volatile("s_mov_b32 m0, %0\n\t" ESMOE_DMA1(2, " nt") ::"s"(lds_addr), "s"(base), "v"(v[0]) : "memory", "m0");
+    else asm volatile("s_mov_b32 m0, %0\n\t" ESMOE_DMA1(2, "") ::"s"(lds_addr), "s"(base), "v"(v[0]) : "memory", "m0");
+  } else if constexpr (N == 2) {
+    if constexpr (NT) asm volatile("s_mov_b32 m0, %0\n\t" ESMOE_DMA1(2, " nt") ESMOE_DMAO(3, 1024, " nt")
+                                   ::"s"(lds_addr), "s"(base), "v"(v[0]), "v"(v[1]) : "memory", "m0");
+    else asm volatile("s_mov_b32 m0, %0\n\t" ESMOE_DMA1(2, "") ESMOE_DMAO(3, 1024, "")
+                      ::"s"(lds_addr), "s"(base), "v"(v[0]), "v"(v[1]) : "memory", "m0");
+  } else if constexpr (N == 3) {
+    if constexpr (NT) asm volatile("s_mov_b32 m0, %0\n\t" ESMOE_DMA1(2, " nt") ESMOE_DMAO(3, 1024, " nt") ESMOE_DMAO(4, 2048, " nt")
+                                   ::"s"(lds_addr), "s"(base), "v"(v[0]), "v"(v[1]), "v"(v[2]) : "memory", "m0");
+    else asm volatile("s_mov_b32 m0, %0\n\t" ESMOE_DMA1(2, "") ESMOE_DMAO(3, 1024, "") ESMOE_DMAO(4, 2048, "")
+                      ::"s"(lds_addr), "s"(base), "v"(v[0]), "v"(v[1]), "v"(v[2]) : "memory", "m0");
+  } else {
+    if constexpr (NT) asm volatile("s_mov_b32 m0, %0\n\t" ESMOE_DMA1(2, " nt") ESMOE_DMAO(3, 1024, " nt") ESMOE_DMAO(4, 2048, " nt")
+                                   ESMOE_DMAO(5, 3072, " nt")
+                                   ::"s"(lds_addr), "s"(base), "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]) : "memory", "m0");
+    else asm volatile("s_mov_b32 m0, %0\n\t" ESMOE_DMA1(2, "") ESMOE_DMAO(3, 1024, "") ESMOE_DMAO(4, 2048, "") ESMOE_DMAO(5, 3072, "")
+                      ::"s"(lds_addr), "s"(base), "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]) : "memory", "m0");
+  }
 }
-__device__ __forceinline__ void dma16x3(uint32_t lds_addr, const void* b0, uint32_t v0, const void* b1, uint32_t v1,
-                                        const void* b2, uint32_t v2) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %3, %4 offset:1024\n\t"
-               "global_load_lds_dwordx4 %5, %6 offset:2048"
-               ::"s"(lds_addr), "v"(v0), "s"(b0), "v"(v1), "s"(b1), "v"(v2), "s"(b2) : "memory", "m0");
-}
-__device__ __forceinline__ void dma16x4(uint32_t lds_addr, const void* b0, uint32_t v0, const void* b1, uint32_t v1,
-                                        const void* b2, uint32_t v2, const void* b3, uint32_t v3) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %3, %4 offset:1024\n\t"
-               "global_load_lds_dwordx4 %5, %6 offset:2048\n\tglobal_load_lds_dwordx4 %7, %8 offset:3072"
-               ::"s"(lds_addr), "v"(v0), "s"(b0), "v"(v1), "s"(b1), "v"(v2), "s"(b2), "v"(v3), "s"(b3) : "memory", "m0");
-}
-// The same with the non-temporal hint, for lines that no other tile will read again (the weights of an expert that is
-// one tile high): they leave L2 to the operands that are shared.  C2, all such tiles, runs 8 % faster with it.
-__device__ __forceinline__ void dma16x4_nt(uint32_t lds_addr, const void* b0, uint32_t v0, const void* b1, uint32_t v1,
-                                        const void* b2, uint32_t v2, const void* b3, uint32_t v3) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt\n\tglobal_load_lds_dwordx4 %3, %4 offset:1024 nt\n\t"
-               "global_load_lds_dwordx4 %5, %6 offset:2048 nt\n\tglobal_load_lds_dwordx4 %7, %8 offset:3072 nt"
-               ::"s"(lds_addr), "v"(v0), "s"(b0), "v"(v1), "s"(b1), "v"(v2), "s"(b2), "v"(v3), "s"(b3) : "memory", "m0");
-}
+// The non-temporal form (NT) is for lines that no other tile will read again (the weights of an expert that is one
+// tile high): they leave L2 to the operands that are shared.  C2, all such tiles, runs 8 % faster with it.
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0) ; explicit" ::"n"(N) : "memory");
@@ -173,8 +179,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // first row goes into the wave-uniform base.  Blocks that cross the end of the expert's rows
   // take a slower path that clamps the row per lane.
   const int crow = lane >> 3, cslot = lane & 7;
-  const uint32_t ro_even = (uint32_t)crow * (uint32_t)K + ((cslot ^ (crow >> 1)) << 4);
-  const uint32_t ro_odd = ro_even ^ 64u;
   const uint8_t* a_base = (const uint8_t*)g.a + (row_base + m0) * K;
   const uint8_t* w_base = (const uint8_t*)g.b + ((long)e * N + (FUSE ? 0 : n0)) * K;
   const int a_last = M - 1 - m0;   // last valid token row of the tile
@@ -211,49 +215,39 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   auto issue_sa_chunk = [&](int c) { dma16(sc_base + (long)c * 16, scoff, lds0 + sclds + (c & 1) * 4096); };
   // copies of K block kb into ring slot buf: this wavefront's token blocks (consecutive 8-row blocks
   // wave*kACopies + i; short tiles are copied by several wavefronts), its 4 weight blocks, its share
-  // of the scales
+  // of the scales.  Each copy has a per-lane byte offset from the operand's pointer for the K block: source row
+  // (token rows past the expert's last are replaced by the last, weight blocks past the last weight row by valid
+  // ones) times K, plus the chunk that belongs in the lane's LDS slot, minus the instruction offset i*1024; kBias
+  // keeps the sum non-negative and is taken off the pointers.
+  constexpr int kBias = 3072;
   const int ablk0 = (wave * G::kACopies) % G::kABlocks;
-  const bool a_interior = (ablk0 + G::kACopies) * 8 - 1 <= a_last;
-  const uint32_t ro_a0 = (ablk0 & 1) ? ro_odd : ro_even, ro_a1 = ro_a0 ^ 64u;
-  const uint32_t ro_w0 = ro_even, ro_w1 = ro_odd;   // a wavefront's first weight block is even
-  // weight block i of this wavefront, i*1024 already subtracted; blocks past the last weight row are
-  // replaced by valid ones
-  long w_off[G::kWCopies];
+  uint32_t va[G::kACopies], vw[G::kWCopies];
+#pragma unroll
+  for (int i = 0; i < G::kACopies; i++) {
+    const int row = (ablk0 + i) * 8 + crow;
+    const int grow = row > a_last ? a_last : row;
+    va[i] = (uint32_t)grow * (uint32_t)K + (swz(row, cslot) << 4) + kBias - i * 1024;
+  }
 #pragma unroll
   for (int i = 0; i < G::kWCopies; i++) {
     const int blk = wave * G::kWCopies + i;
+    int row;
     if constexpr (FUSE) {
       // LDS rows of wavefront column c (RW rows): RW/2 gate rows of columns n0/2 + c*RW/2 .., then the up rows
       // of the same columns (weight rows I + ...)
       constexpr int kRW = NTW * 16, kBlocks = kRW / 8, kHalfBlocks = kBlocks / 2;
       const int wcol = blk / kBlocks, within = blk % kBlocks;
-      const int row = (within / kHalfBlocks) * (N >> 1) + (n0 >> 1) + wcol * (kRW / 2) + (within % kHalfBlocks) * 8;
-      w_off[i] = (long)row * K - i * 1024;
+      row = (within / kHalfBlocks) * (N >> 1) + (n0 >> 1) + wcol * (kRW / 2) + (within % kHalfBlocks) * 8;
     } else {
-      const int src = n0 + blk * 8 < N ? blk : i;
-      w_off[i] = (long)src * 8 * K - i * 1024;
+      row = (n0 + blk * 8 < N ? blk : i) * 8;
     }
+    vw[i] = (uint32_t)(row + crow) * (uint32_t)K + (swz(blk * 8 + crow, cslot) << 4) + kBias - i * 1024;
   }
+  const uint8_t* a_ptr = a_base - kBias;
+  const uint8_t* w_ptr = w_base - kBias;
   auto issue_a = [&](int kb, int buf) {
     const uint32_t sb = lds0 + buf * G::kStageBytes;
-    const uint8_t* ab = a_base + (long)kb * 128;
-    if (a_interior) {
-      const uint8_t* a0 = ab + (long)ablk0 * 8 * K;
-      const uint32_t la = sb + ablk0 * 1024;
-      const long st = 8L * K - 1024;
-      if constexpr (G::kACopies == 1) dma16(a0, ro_a0, la);
-      else if constexpr (G::kACopies == 2) dma16x2(la, a0, ro_a0, a0 + st, ro_a1);
-      else if constexpr (G::kACopies == 3) dma16x3(la, a0, ro_a0, a0 + st, ro_a1, a0 + 2 * st, ro_a0);
-      else dma16x4(la, a0, ro_a0, a0 + st, ro_a1, a0 + 2 * st, ro_a0, a0 + 3 * st, ro_a1);
-    } else {
-#pragma unroll
-      for (int i = 0; i < G::kACopies; i++) {
-        const int blk = ablk0 + i;
-        int row = blk * 8 + crow;
-        int grow = row > a_last ? a_last : row;
-        dma16(ab, (uint32_t)grow * (uint32_t)K + (swz(row, cslot) << 4), sb + blk * 1024);
-      }
-    }
+    dma16xn<false>(sb + ablk0 * 1024, a_ptr + (long)kb * 128, va);
     if constexpr (!MX) {
       if (!sa4) dma4(sc_base + (long)kb * 4, scoff, sb + sclds);
     } else {
@@ -262,16 +256,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   };
   const bool w_once = m0 == 0 && M <= G::BM;   // the expert is one tile high: nobody else reads these weight rows
   auto issue_w = [&](int kb, int buf) {
-    const uint32_t sb = lds0 + buf * G::kStageBytes;
-    const uint8_t* wb = w_base + (long)kb * 128;
+    const uint32_t lw = lds0 + buf * G::kStageBytes + G::kABytes + wave * G::kWCopies * 1024;
     static_assert(G::kWCopies == 4, "weight copies per wavefront");
-    if (w_once) {
-      dma16x4_nt(sb + G::kABytes + wave * G::kWCopies * 1024, wb + w_off[0], ro_w0, wb + w_off[1], ro_w1, wb + w_off[2], ro_w0,
-                 wb + w_off[3], ro_w1);
-      return;
-    }
-    dma16x4(sb + G::kABytes + wave * G::kWCopies * 1024, wb + w_off[0], ro_w0, wb + w_off[1], ro_w1, wb + w_off[2], ro_w0,
-            wb + w_off[3], ro_w1);
+    if (w_once) dma16xn<true>(lw, w_ptr + (long)kb * 128, vw);
+    else dma16xn<false>(lw, w_ptr + (long)kb * 128, vw);
   };
   auto issue = [&](int kb, int buf) { issue_a(kb, buf); issue_w(kb, buf); };
 
@@ -311,6 +299,91 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     float sb_up;   // FUSE: scale of the up rows' weight block (sb is the gate rows')
   };
 
+  auto read_scales_fp8 = [&](int kb, int buf, Frags& f) {
+    const uint8_t* lb = lds + buf * G::kStageBytes;
+    f.sb = sb_tab[kb];
+    if constexpr (FUSE) f.sb_up = sb_tab[kMaxKB + kb];
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) {
+      f.sc[mt] = sa4 ? *(const float*)(lds + sa4_lane + ((kb >> 2) & 1) * 4096 + (kb & 3) * 4 + mt * 256)
+                     : *(const float*)(lb + sa_lane + mt * 64);
+    }
+  };
+
+  // fp8-blockwise tiles of 128 and 192 rows: the copies of K block kb2 into ring slot nbuf, spread between the
+  // fragment reads of slot buf.  A wavefront that issues its copies back to back sits in the queue to the texture
+  // path (one 1 KB copy per ~18 cycles and CU) for as long as the fragment reads then take; interleaved, the two
+  // overlap.  One statement, so that m0 is written once per operand and nothing is scheduled in between; the
+  // fragment halves are read into separate registers that the register allocator places side by side.
+  constexpr bool kInterleave = !MX && (MT == 8 || MT == 12);
+  auto issue_and_read = [&](int kb2, int nbuf, int kb, int buf, Frags& f) {
+    if constexpr (kInterleave) {
+      static_assert(NTW == 4 && G::kWCopies == 4 && kPre == MTW, "interleaved issue: wavefront shape");
+      const uint32_t sbn = lds0 + nbuf * G::kStageBytes;
+      const uint32_t la = sbn + ablk0 * 1024, lw = sbn + G::kABytes + wave * G::kWCopies * 1024;
+      const uint8_t* ap = a_ptr + (long)kb2 * 128;
+      const uint8_t* wp = w_ptr + (long)kb2 * 128;
+      const uint32_t rb = lds0 + buf * G::kStageBytes;
+      const uint32_t wl = rb + wfrag_lo, wh = rb + (wfrag_lo ^ 64), al = rb + afrag_lo, ah = rb + (afrag_lo ^ 64);
+      v4i w0l, w0h, w1l, w1h, w2l, w2h, w3l, w3h, a0l, a0h, a1l, a1h, a2l, a2h, a3l, a3h;
+#define ESMOE_RD(dst, addr, off) "ds_read_b128 %[" #dst "], %[" #addr "] offset:" #off "\n\t"
+#define ESMOE_CP(v, base, off, nt) "global_load_lds_dwordx4 %[" #v "], %[" #base "] offset:" #off nt "\n\t"
+#define ESMOE_OUT(x) [x] "=&v"(x)
+#define ESMOE_FRAG_OUTS                                                                                                     \
+  ESMOE_OUT(w0l), ESMOE_OUT(w0h), ESMOE_OUT(w1l), ESMOE_OUT(w1h), ESMOE_OUT(w2l), ESMOE_OUT(w2h), ESMOE_OUT(w3l), ESMOE_OUT(w3h), \
+  ESMOE_OUT(a0l), ESMOE_OUT(a0h), ESMOE_OUT(a1l), ESMOE_OUT(a1h), ESMOE_OUT(a2l), ESMOE_OUT(a2h), ESMOE_OUT(a3l), ESMOE_OUT(a3h)
+#define ESMOE_COMMON_INS                                                                                                    \
+  [la] "s"(la), [lw] "s"(lw), [ap] "s"(ap), [wp] "s"(wp), [va0] "v"(va[0]), [va1] "v"(va[1]), [vw0] "v"(vw[0]), [vw1] "v"(vw[1]), \
+  [vw2] "v"(vw[2]), [vw3] "v"(vw[3]), [wl] "v"(wl), [wh] "v"(wh), [al] "v"(al), [ah] "v"(ah)
+      if constexpr (MT == 8) {
+#define ESMOE_BODY8(nt)                                                                                                     \
+  "s_mov_b32 m0, %[la]\n\t"                                                                                                 \
+  ESMOE_CP(va0, ap, 0, "") ESMOE_RD(w0l, wl, 0) ESMOE_RD(w0h, wh, 0) ESMOE_RD(a0l, al, 0)                                   \
+  ESMOE_CP(va1, ap, 1024, "") ESMOE_RD(a0h, ah, 0) ESMOE_RD(w1l, wl, 2048) ESMOE_RD(w1h, wh, 2048)                          \
+  "s_mov_b32 m0, %[lw]\n\t"                                                                                                 \
+  ESMOE_CP(vw0, wp, 0, nt) ESMOE_RD(a1l, al, 2048) ESMOE_RD(a1h, ah, 2048) ESMOE_RD(w2l, wl, 4096)                          \
+  ESMOE_CP(vw1, wp, 1024, nt) ESMOE_RD(w2h, wh, 4096) ESMOE_RD(a2l, al, 4096) ESMOE_RD(a2h, ah, 4096)                       \
+  ESMOE_CP(vw2, wp, 2048, nt) ESMOE_RD(w3l, wl, 6144) ESMOE_RD(w3h, wh, 6144) ESMOE_RD(a3l, al, 6144)                       \
+  ESMOE_CP(vw3, wp, 3072, nt) ESMOE_RD(a3h, ah, 6144)                                                                       \
+  "s_waitcnt lgkmcnt(0)"
+        if (w_once) asm volatile(ESMOE_BODY8(" nt") : ESMOE_FRAG_OUTS : ESMOE_COMMON_INS : "memory", "m0");
+        else asm volatile(ESMOE_BODY8("") : ESMOE_FRAG_OUTS : ESMOE_COMMON_INS : "memory", "m0");
+#undef ESMOE_BODY8
+      } else {
+        v4i a4l, a4h, a5l, a5h;
+#define ESMOE_BODY12(nt)                                                                                                    \
+  "s_mov_b32 m0, %[la]\n\t"                                                                                                 \
+  ESMOE_CP(va0, ap, 0, "") ESMOE_RD(w0l, wl, 0) ESMOE_RD(w0h, wh, 0) ESMOE_RD(a0l, al, 0)                                   \
+  ESMOE_CP(va1, ap, 1024, "") ESMOE_RD(a0h, ah, 0) ESMOE_RD(w1l, wl, 2048) ESMOE_RD(w1h, wh, 2048)                          \
+  ESMOE_CP(va2, ap, 2048, "") ESMOE_RD(a1l, al, 2048) ESMOE_RD(a1h, ah, 2048) ESMOE_RD(w2l, wl, 4096)                       \
+  "s_mov_b32 m0, %[lw]\n\t"                                                                                                 \
+  ESMOE_CP(vw0, wp, 0, nt) ESMOE_RD(w2h, wh, 4096) ESMOE_RD(a2l, al, 4096) ESMOE_RD(a2h, ah, 4096)                          \
+  ESMOE_CP(vw1, wp, 1024, nt) ESMOE_RD(w3l, wl, 6144) ESMOE_RD(w3h, wh, 6144) ESMOE_RD(a3l, al, 6144)                       \
+  ESMOE_CP(vw2, wp, 2048, nt) ESMOE_RD(a3h, ah, 6144) ESMOE_RD(a4l, al, 8192) ESMOE_RD(a4h, ah, 8192)                       \
+  ESMOE_CP(vw3, wp, 3072, nt) ESMOE_RD(a5l, al, 10240) ESMOE_RD(a5h, ah, 10240)                                             \
+  "s_waitcnt lgkmcnt(0)"
+        if (w_once)
+          asm volatile(ESMOE_BODY12(" nt") : ESMOE_FRAG_OUTS, ESMOE_OUT(a4l), ESMOE_OUT(a4h), ESMOE_OUT(a5l), ESMOE_OUT(a5h)
+                       : ESMOE_COMMON_INS, [va2] "v"(va[G::kACopies - 1]) : "memory", "m0");
+        else
+          asm volatile(ESMOE_BODY12("") : ESMOE_FRAG_OUTS, ESMOE_OUT(a4l), ESMOE_OUT(a4h), ESMOE_OUT(a5l), ESMOE_OUT(a5h)
+                       : ESMOE_COMMON_INS, [va2] "v"(va[G::kACopies - 1]) : "memory", "m0");
+#undef ESMOE_BODY12
+        f.af[kPre - 2] = join(a4l, a4h);
+        f.af[kPre - 1] = join(a5l, a5h);
+      }
+#undef ESMOE_RD
+#undef ESMOE_CP
+#undef ESMOE_OUT
+#undef ESMOE_FRAG_OUTS
+#undef ESMOE_COMMON_INS
+      f.wf[0] = join(w0l, w0h); f.wf[1] = join(w1l, w1h); f.wf[2] = join(w2l, w2h); f.wf[3] = join(w3l, w3h);
+      f.af[0] = join(a0l, a0h); f.af[1] = join(a1l, a1h); f.af[2] = join(a2l, a2h); f.af[3] = join(a3l, a3h);
+      if (!sa4) dma4(sc_base + (long)kb2 * 4, scoff, sbn + sclds);
+      read_scales_fp8(kb, buf, f);
+    }
+  };
+
   auto read_phase = [&](int kb, int buf, Frags& f) {
     const uint8_t* lb = lds + buf * G::kStageBytes;
 #pragma unroll
@@ -347,13 +420,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
         f.sfa[mt] = (int)(d >> (gq * 8));
       }
     } else {
-      f.sb = sb_tab[kb];
-      if constexpr (FUSE) f.sb_up = sb_tab[kMaxKB + kb];
-#pragma unroll
-      for (int mt = 0; mt < MTW; mt++) {
-        f.sc[mt] = sa4 ? *(const float*)(lds + sa4_lane + ((kb >> 2) & 1) * 4096 + (kb & 3) * 4 + mt * 256)
-                       : *(const float*)(lb + sa_lane + mt * 64);
-      }
+      read_scales_fp8(kb, buf, f);
     }
   };
 
@@ -512,9 +579,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       issue_sa_chunk((kb >> 2) + 1);
       chunk_age = 0;
     }
-    if (more) { if constexpr (kSplitIssue) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
     __builtin_amdgcn_sched_barrier(0);
-    read_phase(kb, buf, f);
+    if (kInterleave && more) {
+      issue_and_read(kb + NBUF - 1, nbuf, kb, buf, f);
+    } else {
+      if (more) { if constexpr (kSplitIssue) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
+      __builtin_amdgcn_sched_barrier(0);
+      read_phase(kb, buf, f);
+    }
     __builtin_amdgcn_sched_barrier(0);
     if (grp == 1) wait_stage(more, chunk_age < NBUF - 2);
     if constexpr (kPP) block_barrier();
