@@ -20,7 +20,7 @@ import torch
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "gemm"): 1.386e9,     # FETCH 650,196.3 x 2.000 KiB + WRITE 52,815.2 x 1.000 KiB
+    ("c1", "gemm"): 1.388e9,     # FETCH 650,196.3 x 2.000 KiB + WRITE 52,815.2 x 1.000 KiB
     ("c4", "quant"): 1.786e8,    # FETCH 57,399.6 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
 }
 
