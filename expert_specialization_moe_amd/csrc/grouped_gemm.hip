@@ -41,6 +41,7 @@
 #include <stdint.h>
 
 #include "gemm_args.h"
+#include "mx_phase.h"
 #include "schedule.h"
 
 namespace esmoe {
@@ -294,7 +295,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // the matrix pipe busy, the other group reads its fragments from LDS.
   //   read phase: weight fragments, the first kPre token fragments and all scales -> registers
   //   mfma phase: the MFMAs (+ the fp32 promotion for fp8-blockwise) of the K block
-  constexpr int kPre = MTW < 4 ? MTW : (MTW == 6 ? 6 : 4);
+  // (256-row mxfp8 tiles read only the first token fragment there: their MFMA phase is one hand-scheduled statement
+  // that fetches row tile mt + 1 under the MFMAs of mt and sends the next stage's copies between the MFMAs, see
+  // mx_phase.h.  All eight wavefronts run that phase at the same time, and issued in one burst at the top of the K
+  // block their 72 copies occupied the texture path for ~1000 cycles in which no MFMA ran.)
+  constexpr bool kMx256 = MX && MT == 16;
+  constexpr int kPre = kMx256 ? 1 : MTW < 4 ? MTW : (MTW == 6 ? 6 : 4);
   struct Frags {
     v8i wf[NTW];
     v8i af[kPre];
@@ -430,6 +436,21 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     }
   };
 
+  // 256-row mxfp8 tiles: the whole phase is the statement of mx_phase.h.
+  // One statement for every K block, so that the accumulators keep their registers around the loop: past the last
+  // K block that has a stage to fetch, the copies fetch the last K block once more into the slot that is free anyway.
+  auto mfma_phase_mx = [&](int buf, const Frags& f, int kb2, int slot) {
+    if constexpr (kMx256) {
+      const uint32_t rb = lds0 + buf * G::kStageBytes;
+      const uint32_t al = rb + afrag_lo, ah = rb + (afrag_lo ^ 64);
+      const uint32_t sbn = lds0 + slot * G::kStageBytes;
+      const uint32_t la = sbn + ablk0 * 1024, lw = sbn + G::kABytes + wave * G::kWCopies * 1024, ls = sbn + sclds;
+      const uint8_t* ap = a_ptr + (long)kb2 * 128;
+      const uint8_t* wp = w_ptr + (long)kb2 * 128;
+      const uint8_t* sp = sc_base + (long)kb2 * 512;
+      asm volatile(ESMOE_MX256_PHASE : ESMOE_MX256_OUTS : ESMOE_MX256_INS : ESMOE_MX256_CLOBBERS);
+    }
+  };
   // fp8-blockwise with all fragments in registers: MFMAs and promotions form one scheduling region in which
   // the four v_fmac of MFMA j - 3 follow MFMA j, so the vector ALU works in the shadow of the matrix pipe
   // and no promotion waits on the MFMA it has just been issued behind.  Taller tiles (fragments read from
@@ -589,7 +610,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     if (kInterleave && more) {
       issue_and_read(kb + NBUF - 1, nbuf, kb, buf, f);
     } else {
-      if (more) { if constexpr (kSplitIssue) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
+      if (more) { if constexpr (kSplitIssue) issue_a(kb + NBUF - 1, nbuf); else if constexpr (!kMx256) issue(kb + NBUF - 1, nbuf); }
       __builtin_amdgcn_sched_barrier(0);
       read_phase(kb, buf, f);
     }
@@ -601,7 +622,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       else if (kb + NBUF < KB) issue_w(kb + NBUF, buf);
     }
     __builtin_amdgcn_sched_barrier(0);
-    mfma_phase(buf, f);
+    if constexpr (kMx256) mfma_phase_mx(buf, f, more ? kb + NBUF - 1 : KB - 1, nbuf);
+    else mfma_phase(buf, f);
     __builtin_amdgcn_sched_barrier(0);
     if (grp == 0) wait_stage(more, chunk_age < NBUF - 2);
     chunk_age++;
