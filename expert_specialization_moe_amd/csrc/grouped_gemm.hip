@@ -842,7 +842,10 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     const int local = v - first;
     TileCoord t;
     if (light) t = sched_decode_light(local, M, g.policy);
-    else if (!sched_decode_heavy(local, ticket % kBlkTiles, M, g.n, g.policy, &t)) continue;
+    else if (!sched_decode_heavy(local, ticket % kBlkTiles, M, g.n, g.policy, &t)) {
+      __syncthreads();   // s_item is rewritten next: every wavefront must have read this ticket first
+      continue;
+    }
 #ifdef ESMOE_TIMELINE
     const uint64_t tl_t0 = __builtin_amdgcn_s_memrealtime();
 #endif
