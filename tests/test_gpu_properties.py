@@ -80,12 +80,16 @@ def test_power_of_two_scale_shift_and_expert_permutation(esmoe):
     assert torch.equal(y3, y1)
 
 
-@pytest.mark.parametrize("cfg", ["c1", "c2"])
+@pytest.mark.parametrize("cfg", ["c1", "c2", "c3:512:zipf", "c3:2048:uniform"])
 def test_benchmark_shapes_sampled_against_oracle(esmoe, cfg):
     """Real shapes of the benchmark configurations; the oracle checks a sample of experts and columns."""
     from expert_specialization_moe_amd import workloads as W
 
-    prob = W.config_problem(cfg, seed=0)
+    if cfg.startswith("c3"):
+        _, tokens, routing = cfg.split(":")
+        prob = W.config_problem("c3", seed=0, tokens=int(tokens), routing=routing)
+    else:
+        prob = W.config_problem(cfg, seed=0)
     ops = W.make_fp8_blockwise_operands(prob, "cuda", seed=0)
     ops["output"].fill_(float("nan"))
     esmoe.es_fp8_blockwise_scaled_grouped_mm(ops["output"], ops["a"], ops["b"], ops["scales_a"], ops["scales_b"],
@@ -109,6 +113,49 @@ def test_benchmark_shapes_sampled_against_oracle(esmoe, cfg):
         ref = ofp8.grouped_mm(a, b, sa, sb, [[len(rows_idx), 384, prob.k]], [0])
         y = H.f32(out[off:off + m, cols])[rows_idx]
         H.check_close(y, ref, f"{cfg} expert {e}")
+
+
+def test_c4_shape_quant_bit_exact_and_gemm_sampled_against_oracle(esmoe):
+    """MXFP8 benchmark configuration at its real size: stage 1 (grouped quantisation of activations, and of the weights
+    through the transposed problem list) bit-exact and stage 2 (block-scaled GEMM) within tolerance, on a sample of
+    experts, rows and columns that the oracle finishes in seconds."""
+    from expert_specialization_moe_amd import workloads as W
+    from oracle import mxfp8 as omx
+
+    prob = W.config_problem("c4", seed=0)
+    ops = W.make_mxfp8_operands(prob, "cuda", seed=0)
+    ops["output"].fill_(float("nan"))
+    esmoe.es_sm100_mxfp8_blockscaled_grouped_mm(ops["output"], ops["a"], ops["b"], ops["sfa"], ops["sfb"],
+                                                ops["problem_sizes"], ops["expert_offsets"], ops["blockscale_offsets"])
+    torch.cuda.synchronize()
+    out = ops["output"]
+    assert not torch.isnan(out).any()
+    n, k, kc = prob.n, prob.k, prob.k // 32
+    offs = W.offsets_of(prob.rows)
+    bso = ops["blockscale_offsets"].cpu().numpy()
+    sfa_flat = ops["sfa"].cpu().numpy().reshape(-1)
+    order = np.argsort(prob.rows)
+    for e in [int(order[-1]), int(order[len(order) // 2]), int(order[0])]:
+        m, off = prob.rows[e], int(offs[e])
+        rows_idx = np.unique(np.concatenate([np.arange(min(200, m)), np.arange(max(0, m - 40), m)]))
+        cols = slice(n - 384, n)
+        # stage 1, activations: bytes and scale codes of the sampled rows
+        x = H.hp_to_f32(ops["a_hp"][off:off + m].cpu())[rows_idx]
+        q_ref, sc_ref = omx.quant_rows(x)
+        a_codes = H.codes(ops["a"][off:off + m])[rows_idx]
+        sa = omx.unswizzle_scales(sfa_flat, m, k, base=int(bso[e]) * kc)[rows_idx]
+        assert np.array_equal(a_codes, q_ref) and np.array_equal(sa, sc_ref), f"c4 activation quant, expert {e}"
+        # stage 1, weights: the last 384 weight rows of the expert
+        w = H.hp_to_f32(ops["w_hp"][e * n + n - 384:(e + 1) * n].cpu())
+        wq_ref, wsc_ref = omx.quant_rows(w)
+        b_codes = H.codes(ops["b_phys"][e, cols])
+        sb = omx.unswizzle_scales(ops["sfb_phys"][e].cpu().numpy().reshape(-1), n, k)[cols]
+        assert np.array_equal(b_codes, wq_ref) and np.array_equal(sb, wsc_ref), f"c4 weight quant, expert {e}"
+        # stage 2
+        ref = omx.dequant_rows(a_codes, sa) @ omx.dequant_rows(b_codes, sb).T
+        ref = torch.from_numpy(ref).to(torch.bfloat16).to(torch.float32).numpy()
+        y = H.f32(out[off:off + m, cols])[rows_idx]
+        H.check_close(y, ref, f"c4 expert {e}")
 
 
 def test_reference_style_diff_against_unquantised_product(esmoe):
