@@ -18,6 +18,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "swiglu.h"
+
 namespace esmoe {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -120,7 +122,7 @@ swiglu_quant_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q, fl
         u0 = __builtin_bit_cast(float, wu << 16);
         u1 = __builtin_bit_cast(float, wu & 0xffff0000u);
       }
-      const float h0 = (g0 / (1.0f + expf(-g0))) * u0, h1 = (g1 / (1.0f + expf(-g1))) * u1;
+      const float h0 = swiglu_f32(g0, u0), h1 = swiglu_f32(g1, u1);
       if constexpr (FP16) {
         x[2 * i] = (float)(_Float16)h0;
         x[2 * i + 1] = (float)(_Float16)h1;

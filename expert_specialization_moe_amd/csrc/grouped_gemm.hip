@@ -43,6 +43,7 @@
 #include "gemm_args.h"
 #include "mx_phase.h"
 #include "schedule.h"
+#include "swiglu.h"
 
 namespace esmoe {
 
@@ -657,7 +658,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
             gv = (float)(__bf16)acc[nt][mt][i];
             uv = (float)(__bf16)acc[nt + kHalf][mt][i];
           }
-          float hv = (gv / (1.0f + expf(-gv))) * uv;
+          float hv = swiglu_f32(gv, uv);
           hv = f16 ? (float)(_Float16)hv : (float)(__bf16)hv;
           h[mt][nt][i] = hv;
           amax = __builtin_fmaxf(amax, __builtin_fabsf(hv));

@@ -24,6 +24,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "swiglu.h"
+
 namespace esmoe {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -120,7 +122,7 @@ __global__ void __launch_bounds__(kQuantThreads) __attribute__((amdgpu_waves_per
       float u[8];
       unpack8<FP16>(rup[p], u);
 #pragma unroll
-      for (int i = 0; i < 8; i++) x[i] = round_to_input_type<FP16>((x[i] / (1.0f + expf(-x[i]))) * u[i]);
+      for (int i = 0; i < 8; i++) x[i] = round_to_input_type<FP16>(swiglu_f32(x[i], u[i]));
     }
     float amax = 0.f;
 #pragma unroll
