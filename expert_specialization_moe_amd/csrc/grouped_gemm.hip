@@ -821,7 +821,13 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     __syncthreads();
     const int ticket = __builtin_amdgcn_readfirstlane(s_item);
     const int kind = light ? kRecItem : kRecBlock;
+#ifdef ESMOE_TIMELINE
+    // (the debug build's extra code keeps the compiler from seeing that this is wave-uniform, and the copies need
+    // their base pointers in scalar registers)
+    const int v = __builtin_amdgcn_readfirstlane(light ? ticket : sched_ticket_block(xq, ticket));
+#else
     const int v = light ? ticket : sched_ticket_block(xq, ticket);
+#endif
     if (v >= (light ? ltotal : hblocks)) {   // this queue is exhausted: the next XCD's, then the other kind
       __syncthreads();                        // s_item is rewritten next
       if (light || ++q == kXcds) {
