@@ -373,12 +373,16 @@ int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int 
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_schedule");
   const esmoe::SchedPolicy p = make_policy(force_bm, 0);
   auto rows_of = [&](int e) { return problem_sizes_host[e * 3] < 0 ? 0 : problem_sizes_host[e * 3]; };
-  // same ranking as the device schedule kernel: most rows first, ties by expert index
+  // same ranking as the device schedule kernel: by sched_order_key, ties by expert index
   for (int e = 0; e < num_experts; e++) {
     int pos = e;
-    if (p.order == 0) {
+    if (p.order != 1) {
       pos = 0;
-      for (int j = 0; j < num_experts; j++) pos += (rows_of(j) > rows_of(e)) || (rows_of(j) == rows_of(e) && j < e);
+      const int key = esmoe::sched_order_key(rows_of(e), p);
+      for (int j = 0; j < num_experts; j++) {
+        const int kj = esmoe::sched_order_key(rows_of(j), p);
+        pos += (kj < key) || (kj == key && j < e);
+      }
     }
     ws_host[esmoe::ws_rec(pos) + esmoe::kRecExpert] = e;
     ws_host[esmoe::ws_rec(pos) + esmoe::kRecRows] = rows_of(e);

@@ -735,11 +735,12 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
   __syncthreads();
   int pos = e;
   if (e < num_experts) {
-    if (policy.order == 0) {
+    if (policy.order != 1) {
       pos = 0;
+      const int key = sched_order_key(m, policy);
       for (int j = 0; j < num_experts; j++) {
-        int mj = s_m[j];
-        pos += (mj > m) || (mj == m && j < e);
+        const int kj = sched_order_key(s_m[j], policy);
+        pos += (kj < key) || (kj == key && j < e);
       }
     }
     ws[ws_rec(pos) + kRecExpert] = e;

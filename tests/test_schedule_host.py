@@ -73,12 +73,13 @@ def test_auto_shapes_waste_less_than_any_single_shape(esmoe):
     assert auto - sum(rows) <= 64 * len(rows)
 
 
-def test_order_is_most_rows_first(esmoe):
+def test_order_is_fewest_rows_first_for_heavy_and_most_rows_first_for_light(esmoe):
     from expert_specialization_moe_amd import _native
 
     rows = [5, 900, 0, 64, 900, 7, 65]
     tiles, origin = _schedule(_native, rows, 256, 0, with_origin=True)
-    # heavy experts (more than 64 rows) in block order, light ones in item order; ties by expert index, empty absent
+    # heavy experts (more than 64 rows) in block order, fewest rows first; light ones in item order, most rows first;
+    # ties by expert index, empty absent
     heavy = sorted((o[2] * 8 + o[1], t[0]) for t, o in zip(tiles, origin) if o[0] == "heavy")
     light = [t[0] for t, o in zip(tiles, origin) if o[0] == "light"]
 
@@ -89,7 +90,7 @@ def test_order_is_most_rows_first(esmoe):
                 r.append(e)
         return r
 
-    assert runs([e for _, e in heavy]) == [1, 4, 6]
+    assert runs([e for _, e in heavy]) == [6, 1, 4]
     assert runs(light) == [3, 5, 0]
 
 
