@@ -26,6 +26,20 @@ namespace esmoe {
 constexpr int kChunk = 1024;       // pairs per wavefront
 constexpr int kMaxRouteExperts = 1024;
 
+// Lanes of the wavefront that hold the same id as this lane: one ballot per bit of the id instead of one round per
+// distinct id (64 pairs over 32 experts are ~25 distinct ids, and a round costs as much as all the ballots together).
+// `bits` covers num_experts - 1; lanes with id < 0 get a meaningless mask.
+__device__ __forceinline__ unsigned long long lanes_with_same_id(int id, int bits) {
+  unsigned long long same = __ballot(id >= 0);
+  for (int b = 0; b < bits; b++) {
+    const bool bit = (id >> b) & 1;
+    const unsigned long long m = __ballot(bit);
+    same &= bit ? m : ~m;
+  }
+  return same;
+}
+__device__ __forceinline__ int id_bits(int num_experts) { return num_experts > 1 ? 32 - __builtin_clz(num_experts - 1) : 0; }
+
 __global__ void __launch_bounds__(64) route_count_kernel(const int* __restrict__ ids, long num_pairs, int first_expert,
                                                          int num_experts, int* __restrict__ chunk_counts) {
   __shared__ int s_cnt[kMaxRouteExperts];
@@ -90,6 +104,7 @@ __global__ void __launch_bounds__(64) route_rank_kernel(const int* __restrict__ 
   for (int e = lane; e < num_experts; e += 64) s_run[e] = expert_offsets[e] + chunk_base[(long)blockIdx.x * num_experts + e];
   __syncthreads();
   const long base = (long)blockIdx.x * kChunk;
+  const int bits = id_bits(num_experts);
   for (int step = 0; step < kChunk / 64; step++) {
     const long p = base + step * 64 + lane;
     if (base + step * 64 >= num_pairs) break;   // wave-uniform
@@ -98,22 +113,14 @@ __global__ void __launch_bounds__(64) route_rank_kernel(const int* __restrict__ 
       id = ids[p] - first_expert;
       if (id < 0 || id >= num_experts) id = -1;
     }
+    // lanes with the same id take consecutive rows in lane order; the first of them moves the expert's counter on
     int row = -1;
-    // group the lanes by id: every round settles the lanes that share the id of the first unsettled lane
-    unsigned long long todo = __ballot(id >= 0);
-    while (todo) {
-      const int leader = __builtin_ctzll(todo);
-      const int lid = __shfl(id, leader);
-      const unsigned long long same = __ballot(id == lid);
-      if (id == lid) {
-        const int before = __builtin_popcountll(same & ((1ull << lane) - 1ull));
-        row = s_run[lid] + before;
-      }
-      __builtin_amdgcn_wave_barrier();
-      if (lane == leader) s_run[lid] += __builtin_popcountll(same);
-      __builtin_amdgcn_wave_barrier();
-      todo &= ~same;
-    }
+    const unsigned long long same = lanes_with_same_id(id, bits);
+    const int before = __builtin_popcountll(same & ((1ull << lane) - 1ull));
+    if (id >= 0) row = s_run[id] + before;
+    __builtin_amdgcn_wave_barrier();
+    if (id >= 0 && before == 0) s_run[id] += __builtin_popcountll(same);
+    __builtin_amdgcn_wave_barrier();
     if (p < num_pairs) dst_row[p] = row;
   }
 }
@@ -174,6 +181,7 @@ __global__ void __launch_bounds__(kSmallChunks * 64) route_small_kernel(const in
     for (int c = 0; c < kSmallChunks; c++) s_cnt[c][tid] += off;
   }
   __syncthreads();
+  const int bits = id_bits(num_experts);
   for (int step = 0; step < kChunk / 64; step++) {
     const long p = base + step * 64 + lane;
     if (base + step * 64 >= num_pairs) break;   // wave-uniform
@@ -183,17 +191,12 @@ __global__ void __launch_bounds__(kSmallChunks * 64) route_small_kernel(const in
       if (id < 0 || id >= num_experts) id = -1;
     }
     int row = -1;
-    unsigned long long todo = __ballot(id >= 0);
-    while (todo) {
-      const int leader = __builtin_ctzll(todo);
-      const int lid = __shfl(id, leader);
-      const unsigned long long same = __ballot(id == lid);
-      if (id == lid) row = s_cnt[w][lid] + __builtin_popcountll(same & ((1ull << lane) - 1ull));
-      __builtin_amdgcn_wave_barrier();
-      if (lane == leader) s_cnt[w][lid] += __builtin_popcountll(same);
-      __builtin_amdgcn_wave_barrier();
-      todo &= ~same;
-    }
+    const unsigned long long same = lanes_with_same_id(id, bits);
+    const int before = __builtin_popcountll(same & ((1ull << lane) - 1ull));
+    if (id >= 0) row = s_cnt[w][id] + before;
+    __builtin_amdgcn_wave_barrier();
+    if (id >= 0 && before == 0) s_cnt[w][id] += __builtin_popcountll(same);
+    __builtin_amdgcn_wave_barrier();
     if (p < num_pairs) dst_row[p] = row;
   }
 }
