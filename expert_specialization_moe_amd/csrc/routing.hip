@@ -66,12 +66,18 @@ __global__ void __launch_bounds__(1024) route_scan_kernel(int* __restrict__ chun
   const int e = threadIdx.x;
   int total = 0;
   if (e < num_experts) {
-    // exclusive scan over the chunks, in place: chunk_counts[c][e] becomes the rank base of chunk c
-    for (int c = 0; c < num_chunks; c++) {
-      const long idx = (long)c * num_experts + e;
-      const int v = chunk_counts[idx];
-      chunk_counts[idx] = total;
-      total += v;
+    // exclusive scan over the chunks, in place: chunk_counts[c][e] becomes the rank base of chunk c.  Sixteen chunks
+    // are read before any is written back, so that a thread waits for memory once per sixteen chunks, not per chunk.
+    constexpr int kBatch = 16;
+    for (int c0 = 0; c0 < num_chunks; c0 += kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; u++) v[u] = c0 + u < num_chunks ? chunk_counts[(long)(c0 + u) * num_experts + e] : 0;
+#pragma unroll
+      for (int u = 0; u < kBatch; u++) {
+        if (c0 + u < num_chunks) chunk_counts[(long)(c0 + u) * num_experts + e] = total;
+        total += v[u];
+      }
     }
     s_cnt[e] = total;
   }
