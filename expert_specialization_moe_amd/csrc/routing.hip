@@ -230,6 +230,34 @@ __global__ void __launch_bounds__(256) permute_rows_kernel(const uint8_t* __rest
   }
 }
 
+// The same packing for topk > 1 (at most 64): one wavefront per token reads the row once and writes it to every
+// local destination of the token's pairs, where one wavefront per pair would read it topk times.
+__global__ void __launch_bounds__(256) permute_rows_by_token_kernel(const uint8_t* __restrict__ in,
+                                                                    const int* __restrict__ dst_row, long num_tokens,
+                                                                    int topk, long row_bytes, uint8_t* __restrict__ out) {
+  typedef int v4i __attribute__((ext_vector_type(4)));
+  const long t = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= num_tokens) return;
+  const int lane = threadIdx.x & 63;
+  const int mine = lane < topk ? dst_row[t * topk + lane] : -1;   // lane j: destination of the token's pair j
+  if (__ballot(mine >= 0) == 0) return;                           // no local pair
+  const uint8_t* src = in + t * row_bytes;
+  for (long off = lane * 16; off < row_bytes; off += 4096) {
+    v4i v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (off + u * 1024 < row_bytes) v[u] = __builtin_nontemporal_load((const v4i*)(src + off + u * 1024));
+    for (int j = 0; j < topk; j++) {
+      const int dst = __builtin_amdgcn_readlane(mine, j);
+      if (dst < 0) continue;
+      uint8_t* d = out + (long)dst * row_bytes;
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        if (off + u * 1024 < row_bytes) __builtin_nontemporal_store(v[u], (v4i*)(d + off + u * 1024));
+    }
+  }
+}
+
 }  // namespace esmoe
 
 extern "C" int esmoe_launch_route_metadata(const int* ids, long num_pairs, int first_expert, int num_experts, int n, int k,
@@ -257,6 +285,12 @@ extern "C" int esmoe_launch_permute_rows(const void* in, const int* dst_row, lon
                                          void* out, hipStream_t stream) {
   using namespace esmoe;
   if (num_pairs == 0) return 0;
+  if (topk > 1 && topk <= 64 && num_pairs % topk == 0) {
+    const long tokens = num_pairs / topk;
+    hipLaunchKernelGGL(permute_rows_by_token_kernel, dim3((unsigned)((tokens + 3) / 4)), dim3(256), 0, stream,
+                       (const uint8_t*)in, dst_row, tokens, topk, row_bytes, (uint8_t*)out);
+    return (int)hipGetLastError();
+  }
   hipLaunchKernelGGL(permute_rows_kernel, dim3((unsigned)((num_pairs + 3) / 4)), dim3(256), 0, stream, (const uint8_t*)in,
                      dst_row, num_pairs, topk, row_bytes, (uint8_t*)out);
   return (int)hipGetLastError();

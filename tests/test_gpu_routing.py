@@ -58,6 +58,24 @@ def test_route_rejects(esmoe):
     assert lib.esmoe_permute_rows(p, p, 4, 1, 24, p, None) == -1
 
 
+@pytest.mark.parametrize("topk,row_elems", [(8, 4096 + 8), (2, 7168), (64, 128), (65, 64), (1, 4104)])
+def test_permute_rows_of_topk_pairs(esmoe, topk, row_elems):
+    """Row packing for top-k routing (a token's row goes to each of its local pairs' rows, remote pairs skipped),
+    rows longer than one 4 KB pass and not a multiple of it; bit-exact against the oracle."""
+    tokens, experts = 77, 96
+    rng = np.random.default_rng(topk)
+    ids = np.stack([rng.permutation(128)[:topk] for _ in range(tokens)]).astype(np.int32)   # experts 96..127 are remote
+    x = torch.randn((tokens, row_elems), generator=torch.Generator().manual_seed(topk)).to(torch.bfloat16)
+    ps, eo, bso, dst = esmoe.es_route_metadata(torch.from_numpy(ids).cuda(), 0, experts, 256, 128)
+    total = int(eo[-1].item())
+    packed = torch.full((total, row_elems), float("nan"), dtype=torch.bfloat16, device="cuda")
+    esmoe.es_permute_rows(x.cuda(), dst, topk, packed)
+    torch.cuda.synchronize()
+    ps_r, eo_r, bso_r, dst_r = oroute.route_metadata(ids, 0, experts, 256, 128)
+    assert np.array_equal(dst.cpu().numpy(), dst_r)
+    assert np.array_equal(H.hp_to_f32(packed.cpu()), oroute.permute_rows(H.hp_to_f32(x), dst_r, topk, total))
+
+
 def test_routed_fp8_layer_on_device(esmoe):
     """ids -> metadata -> packed rows -> 1x128 quant -> grouped GEMM, all on the device, against the oracle chain."""
     from expert_specialization_moe_amd import workloads as W
