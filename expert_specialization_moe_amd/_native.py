@@ -64,11 +64,11 @@ lib.esmoe_last_error.argtypes = []
 lib.esmoe_version.restype = ctypes.c_char_p
 lib.esmoe_version.argtypes = []
 lib.esmoe_host_schedule.restype = _i
-lib.esmoe_host_schedule.argtypes = [_vp, _i, _i, _i, _vp]
+lib.esmoe_host_schedule.argtypes = [_vp, _i, _i, _i, _i, _vp]
 lib.esmoe_host_decode_heavy.restype = _i
-lib.esmoe_host_decode_heavy.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
+lib.esmoe_host_decode_heavy.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp]
 lib.esmoe_host_decode_light.restype = _i
-lib.esmoe_host_decode_light.argtypes = [_vp, _vp, _i, _i, _i, _i, _vp]
+lib.esmoe_host_decode_light.argtypes = [_vp, _vp, _i, _i, _i, _i, _i, _vp]
 
 
 def last_error():

@@ -76,21 +76,60 @@ int current_device_info(DeviceInfo* out) {
   return 0;
 }
 
-int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return v && *v ? atoi(v) : dflt;
+// ESMOE_* environment variables (tuning aids) are read once per process, on the first GEMM launch; a value the
+// kernels cannot honour is reported by every launch instead of being applied.
+struct Knobs {
+  int big_mt_fp8 = 12, big_mt_mx = 16, order = 0, light_share = -1, wgs_per_cu = 1;
+  char error[160] = "";
+};
+
+const Knobs& knobs() {
+  static const Knobs k = [] {
+    Knobs r;
+    auto env_int = [](const char* name, int dflt) {
+      const char* v = getenv(name);
+      return v && *v ? atoi(v) : dflt;
+    };
+    const char* big = getenv("ESMOE_BIG_MT");
+    if (big && *big) {
+      const int v = atoi(big);
+      // mxfp8 tiles of 128 and 256 rows read their token scales assuming a start on a 128-row boundary, which
+      // full tiles of 192 rows would break for the remainder tile: 8 and 16 only.
+      if (v == 8 || v == 16) r.big_mt_fp8 = r.big_mt_mx = v;
+      else if (v == 12) r.big_mt_fp8 = v;
+      else snprintf(r.error, sizeof(r.error), "ESMOE_BIG_MT=%s: full tiles are 8, 12 or 16 x 16 rows (8 or 16 for mxfp8)", big);
+    }
+    r.order = env_int("ESMOE_ORDER", 0);
+    if (r.order < 0 || r.order > 2) snprintf(r.error, sizeof(r.error), "ESMOE_ORDER must be 0, 1 or 2");
+    r.light_share = env_int("ESMOE_LIGHT_SHARE", -1);
+    if (r.light_share < -1 || r.light_share > 32) snprintf(r.error, sizeof(r.error), "ESMOE_LIGHT_SHARE must be in [-1, 32]");
+    r.wgs_per_cu = env_int("ESMOE_WGS_PER_CU", 1);
+    if (r.wgs_per_cu < 1 || r.wgs_per_cu > 8) snprintf(r.error, sizeof(r.error), "ESMOE_WGS_PER_CU must be in [1, 8]");
+    return r;
+  }();
+  return k;
 }
 
-// Default schedule policy; ESMOE_* environment variables override single fields (tuning aid).
-esmoe::SchedPolicy make_policy(int force_bm, int mx) {
+// Default schedule policy: the one the host mirrors describe.
+esmoe::SchedPolicy default_policy(int force_bm, int mx) {
   esmoe::SchedPolicy p;
   p.force_mt = force_bm / 16;
   // Taller tiles do more MFMA work per byte copied into LDS.  The mxfp8 kernel is fastest with 256-row
   // tiles; the fp8-blockwise kernel, whose fp32 promotion shares the vector ALU, gains nothing beyond
   // 192 rows, and shorter full tiles leave less padding in the remainder tile.
-  p.big_mt = env_int("ESMOE_BIG_MT", mx ? 16 : 12);
-  p.order = env_int("ESMOE_ORDER", 0);
-  p.light_share = env_int("ESMOE_LIGHT_SHARE", -1);
+  p.big_mt = mx ? 16 : 12;
+  p.order = 0;
+  p.light_share = -1;
+  return p;
+}
+
+// Policy of a launch: the default with the environment's overrides.
+esmoe::SchedPolicy launch_policy(int force_bm, int mx) {
+  esmoe::SchedPolicy p = default_policy(force_bm, mx);
+  const Knobs& k = knobs();
+  p.big_mt = mx ? k.big_mt_mx : k.big_mt_fp8;
+  p.order = k.order;
+  p.light_share = k.light_share;
   return p;
 }
 
@@ -122,8 +161,9 @@ int launch_gemm(esmoe::GemmArgs& g, int mx, int force_bm, void* stream) {
   DeviceInfo info;
   int rc = current_device_info(&info);
   if (rc) return rc;
-  g.policy = make_policy(force_bm, mx);
-  int grid = info.cus * env_int("ESMOE_WGS_PER_CU", 1);
+  if (knobs().error[0]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "%s", knobs().error);
+  g.policy = launch_policy(force_bm, mx);
+  int grid = info.cus * knobs().wgs_per_cu;
   rc = esmoe_launch_grouped_gemm(&g, mx, grid, (hipStream_t)stream);
   if (rc) return fail(rc, "grouped GEMM launch failed: %s", hipGetErrorString((hipError_t)rc));
   return 0;
@@ -367,11 +407,12 @@ int esmoe_permute_rows(const void* in, const int32_t* dst_row, long num_pairs, i
   return 0;
 }
 
-int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int32_t* ws_host) {
+int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int mx,
+                        int32_t* ws_host) {
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS || n <= 0 || n % 128)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_schedule");
-  const esmoe::SchedPolicy p = make_policy(force_bm, 0);
+  const esmoe::SchedPolicy p = default_policy(force_bm, mx != 0);
   auto rows_of = [&](int e) { return problem_sizes_host[e * 3] < 0 ? 0 : problem_sizes_host[e * 3]; };
   // same ranking as the device schedule kernel: by sched_order_key, ties by expert index
   for (int e = 0; e < num_experts; e++) {
@@ -424,11 +465,11 @@ void fill_out5(int32_t* out5, int e, const esmoe::TileCoord& t) {
 }  // namespace
 
 int esmoe_host_decode_heavy(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                            int force_bm, int xcd, int ticket, int32_t* out5) {
+                            int force_bm, int mx, int xcd, int ticket, int32_t* out5) {
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || !out5 || xcd < 0 || xcd >= esmoe::kXcds || ticket < 0)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_decode_heavy");
-  const esmoe::SchedPolicy p = make_policy(force_bm, 0);
+  const esmoe::SchedPolicy p = default_policy(force_bm, mx != 0);
   const int blk = esmoe::sched_ticket_block(xcd, ticket);
   if (blk >= ws_host[esmoe::kWsHeavyBlocks]) return 2;   // this XCD's queue is exhausted
   const int pos = host_position(ws_host, num_experts, esmoe::kRecBlock, blk);
@@ -442,11 +483,11 @@ int esmoe_host_decode_heavy(const int32_t* problem_sizes_host, const int32_t* ws
 }
 
 int esmoe_host_decode_light(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                            int force_bm, int item, int32_t* out5) {
+                            int force_bm, int mx, int item, int32_t* out5) {
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || !out5) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null pointer");
   (void)n;
-  const esmoe::SchedPolicy p = make_policy(force_bm, 0);
+  const esmoe::SchedPolicy p = default_policy(force_bm, mx != 0);
   if (item < 0 || item >= ws_host[esmoe::kWsLightTotal]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "item out of range");
   const int pos = host_position(ws_host, num_experts, esmoe::kRecItem, item);
   if (pos < 0) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace does not hold a schedule");

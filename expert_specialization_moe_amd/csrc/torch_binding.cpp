@@ -43,8 +43,8 @@ int out_dtype_of(const torch::Tensor& t) { return t.scalar_type() == torch::kBFl
 // enough and aligned, otherwise a small tensor from the caching allocator.
 torch::Tensor schedule_scratch(const torch::Tensor* workspace, int64_t num_experts, const torch::Tensor& like) {
   const int64_t need = (int64_t)esmoe_gemm_workspace_bytes((int)num_experts);
-  if (workspace && workspace->defined() && workspace->is_cuda() && workspace->is_contiguous() &&
-      workspace->nbytes() >= (size_t)need && (reinterpret_cast<uintptr_t>(workspace->data_ptr()) % 16) == 0) {
+  if (workspace && workspace->defined() && workspace->is_cuda() && workspace->device() == like.device() &&
+      workspace->is_contiguous() && workspace->nbytes() >= (size_t)need && (reinterpret_cast<uintptr_t>(workspace->data_ptr()) % 16) == 0) {
     return *workspace;
   }
   return torch::empty({need}, torch::TensorOptions().dtype(torch::kUInt8).device(like.device()));
@@ -198,6 +198,10 @@ void es_sm100_mxfp8_blockscaled_grouped_mm(const torch::Tensor& a, const torch::
               "d must be a contiguous (num_tokens, n) tensor");
   TORCH_CHECK(sfa.element_size() == 1 && sfb.element_size() == 1, "scale factors must be 1-byte E8M0");
   TORCH_CHECK(sfb.numel() >= num_experts * n * (k / 32), "sfb is smaller than num_experts * n * k / 32 bytes");
+  // every expert's scale rows are padded to 128, so the tensor holds at least the row total rounded up (a bound that
+  // needs no look at the device-side metadata)
+  TORCH_CHECK(sfa.numel() >= (total_rows + 127) / 128 * 128 * (k / 32),
+              "sfa is smaller than the rows rounded up to 128 times k / 32 bytes");
   TORCH_CHECK(expert_offsets.dtype() == torch::kInt32 && blockscale_offsets.dtype() == torch::kInt32,
               "offset tensors must be int32");
   TORCH_CHECK(blockscale_offsets.dim() == 1 && blockscale_offsets.size(0) == num_experts,
@@ -251,6 +255,8 @@ void es_sm100_mxfp8_blockscaled_grouped_quant(const torch::Tensor& input, const 
   TORCH_CHECK(scale_factor.is_contiguous() && scale_factor.element_size() == 1,
               "scale_factor must be a contiguous 1-byte tensor");
   const int64_t sf_rows = (scale_factor.numel() / (k / 32)) / 128 * 128;
+  TORCH_CHECK(sf_rows >= (total_rows + 127) / 128 * 128,
+              "scale_factor is smaller than the rows rounded up to 128 times k / 32 bytes");
   TORCH_CHECK(total_rows < (int64_t(1) << 31) && sf_rows < (int64_t(1) << 31), "tensor too large");
 
   require_device(input, "es_sm100_mxfp8_blockscaled_grouped_quant");
@@ -410,6 +416,8 @@ void es_swiglu_mxfp8_grouped_quant(const torch::Tensor& input, const torch::Tens
   TORCH_CHECK(scale_factor.is_contiguous() && scale_factor.element_size() == 1,
               "scale_factor must be a contiguous 1-byte tensor");
   const int64_t sf_rows = (scale_factor.numel() / (inter / 32)) / 128 * 128;
+  TORCH_CHECK(sf_rows >= (total_rows + 127) / 128 * 128,
+              "scale_factor is smaller than the rows rounded up to 128 times inter / 32 bytes");
   TORCH_CHECK(total_rows < (int64_t(1) << 31) && sf_rows < (int64_t(1) << 31), "tensor too large");
   require_device(input, "es_swiglu_mxfp8_grouped_quant");
   for (const torch::Tensor* t : {&problem_sizes, &expert_offsets, &blockscale_offsets, (const torch::Tensor*)&quant_output,

@@ -216,12 +216,16 @@ int esmoe_permute_rows(const void* in, const int32_t* dst_row, long num_pairs, i
  * expert's tile grid (the kernel skips it), or 2 if that XCD's queue is exhausted.
  * The other experts are "light": one short tile per 256 columns from a launch-wide counter;
  * esmoe_host_decode_light maps item `item` (< word 1 of the workspace) to out5.
+ * mx: 0 describes the FP8-blockwise launch (full tiles of 192 rows), 1 the MXFP8 launch (256 rows).  The mirrors
+ * describe the default policy; the ESMOE_* environment variables, which a launch reads once per process, do not
+ * reach them.
  */
-int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int32_t* ws_host);
+int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int mx,
+                        int32_t* ws_host);
 int esmoe_host_decode_heavy(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                            int force_bm, int xcd, int ticket, int32_t* out5);
+                            int force_bm, int mx, int xcd, int ticket, int32_t* out5);
 int esmoe_host_decode_light(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                            int force_bm, int item, int32_t* out5);
+                            int force_bm, int mx, int item, int32_t* out5);
 
 /* Message describing the calling thread's most recent failure ("" if none). */
 const char* esmoe_last_error(void);

@@ -37,6 +37,21 @@ def check_close(y, ref, what=""):
     assert cos >= COS_MIN, f"{what}: cosine {cos}"
 
 
+def check_ulps(y, ref, out_dtype, what="", ulps=2.0, abs_rms=2e-3):
+    """Tight form for a kernel whose accumulation order the oracle follows: every element within `ulps` units in
+    the last place of the output type (bf16: 2^-8 relative, fp16: 2^-11) plus abs_rms of the result's rms, which
+    covers cancellation between K blocks (fp32 sums taken in another order inside a block)."""
+    y = np.asarray(y, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    ok = np.isfinite(ref)
+    eps = 2.0 ** -8 if out_dtype == torch.bfloat16 else 2.0 ** -11
+    rms = np.sqrt((ref[ok] ** 2).mean()) if ok.any() else 0.0
+    err = np.abs(y - ref)[ok]
+    bound = (ulps * eps * np.abs(ref) + abs_rms * rms)[ok]
+    bad = err > bound
+    assert not bad.any(), f"{what}: {bad.sum()} of {bad.size} elements beyond {ulps} ulps, worst ratio {(err / np.maximum(bound, 1e-300)).max():.2f}"
+
+
 def check_grouped(y, ref, rows, offsets, what=""):
     for e, (m, off) in enumerate(zip(rows, offsets)):
         if m:

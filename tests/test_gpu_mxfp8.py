@@ -50,13 +50,13 @@ def test_quant_bit_exact_wide(esmoe):
     _quant_case(esmoe, [513, 64, 0, 0, 1000], 7168, torch.bfloat16, seed=2)
 
 
-@pytest.mark.parametrize("force_bm", [0, 16, 64, 128, 256])
+@pytest.mark.parametrize("force_bm", [0, 16, 32, 64, 128, 192, 256])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
 def test_mx_gemm_parity(esmoe, force_bm, out_dtype):
     from expert_specialization_moe_amd import _native
     from expert_specialization_moe_amd import workloads as W
 
-    prob = W.Problem("ragged", 384, 640, [0, 1, 17, 130, 0, 64, 300, 15, 33], kind="mxfp8")
+    prob = W.Problem("ragged", 384, 640, [0, 1, 17, 130, 0, 64, 300, 15, 33, 530], kind="mxfp8")
     ops = W.make_mxfp8_operands(prob, "cuda", seed=5, out_dtype=out_dtype, weight_std=1.0)
     ops["output"].fill_(float("nan"))
     y = H.f32(H.capi_mx_mm(_native, ops, force_bm=force_bm))
@@ -65,6 +65,7 @@ def test_mx_gemm_parity(esmoe, force_bm, out_dtype):
                          W.offsets_of(prob.rows), ops["blockscale_offsets"].cpu().numpy(),
                          out_dtype="bf16" if out_dtype == torch.bfloat16 else "fp16")
     H.check_grouped(y, ref, prob.rows, W.offsets_of(prob.rows), f"mx bm={force_bm}")
+    H.check_ulps(y, ref, out_dtype, f"mx bm={force_bm}")
     # rows of empty experts / nothing else: every row belongs to an expert here, so no NaN may remain
     assert np.isfinite(y).all()
 
@@ -176,3 +177,66 @@ def test_swiglu_mxfp8_grouped_quant_against_oracle(esmoe, in_dtype):
     esmoe.es_swiglu_mxfp8_grouped_quant(xd, ps_d, eo_d, bso_d, q_o, sf_o)
     assert torch.equal(q_o, q)
     assert np.array_equal(sf_o.cpu().numpy()[mask], sg[mask])
+
+
+def test_reference_callers_two_byte_buffers_give_the_same_bytes(esmoe):
+    """The reference's end-to-end test hands the quant operator zeros_like(bf16 input) buffers, lets it write e4m3 bytes
+    into them and passes those 2-byte tensors on to the GEMM as `a` and `b`
+    (test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:72-101).  Same calls, same dtypes: the bytes written and the
+    GEMM result must equal those of the uint8 / float8 route."""
+    from expert_specialization_moe_amd import workloads as W
+
+    prob = W.Problem("two_byte", 256, 384, [77, 0, 200, 3, 129], kind="mxfp8")
+    ops = W.make_mxfp8_operands(prob, "cuda", seed=17, weight_std=1.0)
+    e, n, k, total = prob.num_experts, prob.n, prob.k, prob.total_rows
+    a, w = ops["a_hp"], ops["w_hp"]
+    a_quant = torch.zeros_like(a)                      # bf16 [rows, k]: twice the bytes needed
+    b_quant = torch.zeros_like(w)                      # bf16 [e * n, k]
+    sfa = torch.zeros_like(ops["sfa"])
+    sfb = torch.zeros((e, n, k // 32), dtype=torch.uint8, device="cuda")
+    esmoe.es_sm100_mxfp8_blockscaled_grouped_quant(a, ops["problem_sizes"], ops["expert_offsets"], ops["blockscale_offsets"],
+                                                   a_quant, sfa)
+    esmoe.es_sm100_mxfp8_blockscaled_grouped_quant(w, ops["aux_problem_sizes"], ops["aux_expert_offsets"],
+                                                   ops["aux_expert_offsets"], b_quant, sfb)
+    torch.cuda.synchronize()
+    a_bytes = a_quant.view(torch.uint8).reshape(-1)[: total * k].reshape(total, k)
+    b_bytes = b_quant.view(torch.uint8).reshape(-1)[: e * n * k].reshape(e, n, k)
+    assert torch.equal(a_bytes, ops["a"].view(torch.uint8)) and torch.equal(b_bytes, ops["b_phys"].view(torch.uint8))
+    assert torch.equal(sfa, ops["sfa"]) and torch.equal(sfb, ops["sfb_phys"])
+    # the untouched second half of the 2-byte buffers stays zero
+    assert not a_quant.view(torch.uint8).reshape(-1)[total * k:].any()
+    want = torch.empty_like(ops["output"])
+    esmoe.es_sm100_mxfp8_blockscaled_grouped_mm(want, ops["a"], ops["b"], ops["sfa"], ops["sfb"], ops["problem_sizes"],
+                                                ops["expert_offsets"], ops["blockscale_offsets"])
+    got = torch.full_like(want, float("nan"))
+    # the reference reshapes the 2-byte weight buffer to (e, n, k) and hands over its (e, k, n) view
+    esmoe.es_sm100_mxfp8_blockscaled_grouped_mm(got, a_quant, b_quant.view(e, n, k).transpose(1, 2), sfa,
+                                                sfb.view(e, n, k // 32).transpose(1, 2), ops["problem_sizes"],
+                                                ops["expert_offsets"], ops["blockscale_offsets"])
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
+def test_grouped_quant_through_the_c_abi(esmoe):
+    """esmoe_mxfp8_grouped_quant called through ctypes (the other quant tests go through the torch operator)."""
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import workloads as W
+
+    rows, k = [5, 0, 200, 128, 1], 256
+    total = sum(rows)
+    x = torch.randn((total, k), generator=torch.Generator().manual_seed(4)).to(torch.float16)
+    xd = x.cuda()
+    ps = [[m, 11, k] for m in rows]
+    bso_np, sf_rows = W.blockscale_offsets_of(rows)
+    ps_d = torch.tensor(ps, dtype=torch.int32, device="cuda")
+    eo_d = torch.tensor(W.offsets_of(rows), dtype=torch.int32, device="cuda")
+    bso_d = torch.tensor(bso_np, dtype=torch.int32, device="cuda")
+    q = torch.full((total, k), 0x55, dtype=torch.uint8, device="cuda")
+    sf = torch.full((sf_rows * (k // 32),), 0xEE, dtype=torch.uint8, device="cuda")
+    rc = _native.lib.esmoe_mxfp8_grouped_quant(H.ptr(xd), 1, H.ptr(ps_d), H.ptr(eo_d), H.ptr(bso_d), H.ptr(q), H.ptr(sf), len(rows),
+                                               total, sf_rows, k, H.stream_ptr())
+    assert rc == 0, _native.last_error()
+    torch.cuda.synchronize()
+    q_ref, sf_ref, mask = omx.grouped_quant(H.hp_to_f32(x), ps, W.offsets_of(rows), bso_np, sf_total_rows=sf_rows)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    assert np.array_equal(sf.cpu().numpy()[mask], sf_ref[mask])

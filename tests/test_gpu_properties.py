@@ -80,7 +80,7 @@ def test_power_of_two_scale_shift_and_expert_permutation(esmoe):
     assert torch.equal(y3, y1)
 
 
-@pytest.mark.parametrize("cfg", ["c1", "c2", "c3:512:zipf", "c3:2048:uniform"])
+@pytest.mark.parametrize("cfg", ["c1", "c2"] + [f"c3:{t}:{r}" for t in (64, 512, 2048, 8192, 16384) for r in ("zipf", "uniform")])
 def test_benchmark_shapes_sampled_against_oracle(esmoe, cfg):
     """Real shapes of the benchmark configurations; the oracle checks a sample of experts and columns."""
     from expert_specialization_moe_amd import workloads as W

@@ -5,14 +5,14 @@ import numpy as np
 import pytest
 
 
-def _schedule(native, rows, n, force_bm=0, with_origin=False):
+def _schedule(native, rows, n, force_bm=0, with_origin=False, mx=0):
     """Every tile the kernel would compute: all tickets of the 8 per-XCD queues, then the light items."""
     lib = native.lib
     e = len(rows)
     ps = np.array([[m, n, 512] for m in rows], dtype=np.int32)
     ws = np.zeros(lib.esmoe_gemm_workspace_bytes(e) // 4, dtype=np.int32)
     psp, wsp = ps.ctypes.data_as(ctypes.c_void_p), ws.ctypes.data_as(ctypes.c_void_p)
-    rc = lib.esmoe_host_schedule(psp, e, n, force_bm, wsp)
+    rc = lib.esmoe_host_schedule(psp, e, n, force_bm, mx, wsp)
     assert rc == 0, native.last_error()
     light_total, heavy_blocks = int(ws[1]), int(ws[2])
     tiles, origin = [], []
@@ -21,7 +21,7 @@ def _schedule(native, rows, n, force_bm=0, with_origin=False):
     for xcd in range(8):
         ticket = 0
         while True:
-            rc = lib.esmoe_host_decode_heavy(psp, wsp, e, n, force_bm, xcd, ticket, out.ctypes.data_as(ctypes.c_void_p))
+            rc = lib.esmoe_host_decode_heavy(psp, wsp, e, n, force_bm, mx, xcd, ticket, out.ctypes.data_as(ctypes.c_void_p))
             assert rc in (0, 1, 2), native.last_error()
             if rc == 2:
                 break
@@ -33,20 +33,21 @@ def _schedule(native, rows, n, force_bm=0, with_origin=False):
         seen_blocks += ticket // 32
     assert seen_blocks == heavy_blocks
     for item in range(light_total):
-        rc = lib.esmoe_host_decode_light(psp, wsp, e, n, force_bm, item, out.ctypes.data_as(ctypes.c_void_p))
+        rc = lib.esmoe_host_decode_light(psp, wsp, e, n, force_bm, mx, item, out.ctypes.data_as(ctypes.c_void_p))
         assert rc == 0, native.last_error()
         tiles.append(tuple(int(v) for v in out))
         origin.append(("light", item))
     return (tiles, origin) if with_origin else tiles
 
 
+@pytest.mark.parametrize("mx", [0, 1])
 @pytest.mark.parametrize("force_bm", [0, 16, 32, 64, 128, 192, 256])
 @pytest.mark.parametrize("n", [128, 384, 4096])
-def test_tiles_cover_every_output_element_exactly_once(esmoe, force_bm, n):
+def test_tiles_cover_every_output_element_exactly_once(esmoe, force_bm, n, mx):
     from expert_specialization_moe_amd import _native
 
-    rows = [0, 1, 16, 17, 127, 128, 129, 300, 0, 1000, 64, 33]
-    tiles = _schedule(_native, rows, n, force_bm)
+    rows = [0, 1, 16, 17, 127, 128, 129, 300, 0, 1000, 64, 33, 449, 577]
+    tiles = _schedule(_native, rows, n, force_bm, mx=mx)
     cover = [np.zeros((m, n), dtype=np.int32) for m in rows]
     for e, bm, bn, m0, n0 in tiles:
         assert bn == 256 and bm in (16, 32, 64, 128, 192, 256)
@@ -54,8 +55,23 @@ def test_tiles_cover_every_output_element_exactly_once(esmoe, force_bm, n):
         if force_bm:
             assert bm == force_bm
         cover[e][m0:m0 + bm, n0:n0 + bn] += 1
+        if not force_bm:
+            # full tiles: 192 rows for fp8-blockwise, 256 for mxfp8, then one remainder tile
+            assert bm <= (256 if mx else 192)
+            assert m0 % (256 if mx else 192) == 0
+        if mx and bm in (128, 256):
+            # the mxfp8 kernel reads the token scales of these heights assuming a start on a scale-tile boundary
+            assert m0 % 128 == 0
     for c in cover:
         assert (c == 1).all()
+
+
+def test_mx_policy_uses_256_row_full_tiles(esmoe):
+    from expert_specialization_moe_amd import _native
+
+    heights = lambda mx: sorted({t[1] for t in _schedule(_native, [700], 256, 0, mx=mx)})
+    assert heights(0) == [128, 192]      # 3 x 192 + 124 -> 128
+    assert heights(1) == [192, 256]      # 2 x 256 + 188 -> 192
 
 
 def test_auto_shapes_waste_less_than_any_single_shape(esmoe):
