@@ -36,6 +36,8 @@ lib.esmoe_gemm_workspace_bytes.restype = _sz
 lib.esmoe_gemm_workspace_bytes.argtypes = [_i]
 lib.esmoe_fp8_blockwise_grouped_mm.restype = _i
 lib.esmoe_fp8_blockwise_grouped_mm.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]
+lib.esmoe_fp8_blockwise_grouped_mm_static.restype = _i
+lib.esmoe_fp8_blockwise_grouped_mm_static.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]
 lib.esmoe_mxfp8_grouped_mm.restype = _i
 lib.esmoe_mxfp8_grouped_mm.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]
 lib.esmoe_mxfp8_grouped_quant.restype = _i

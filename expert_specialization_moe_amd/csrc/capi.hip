@@ -14,6 +14,7 @@
 #include "schedule.h"
 
 extern "C" int esmoe_launch_grouped_gemm(const esmoe::GemmArgs* args, int mx, int grid, hipStream_t stream);
+extern "C" int esmoe_static_scratch(int32_t** ptr, size_t* bytes, int* max_experts);
 extern "C" int esmoe_launch_mxfp8_quant(const void* in, int in_dtype, const int* problem_sizes,
                                         const int* expert_offsets, const int* blockscale_offsets, void* q, uint8_t* sf,
                                         int num_experts, long sf_rows, int k, int swiglu, long dense_rows,
@@ -195,6 +196,23 @@ int esmoe_fp8_blockwise_grouped_mm(void* out, int out_dtype, const void* a, cons
   g.ws = (int32_t*)workspace;
   g.num_experts = num_experts; g.total_rows = total_rows; g.n = n; g.k = k; g.out_dtype = out_dtype;
   return launch_gemm(g, 0, force_bm, stream);
+}
+
+int esmoe_fp8_blockwise_grouped_mm_static(void* out, int out_dtype, const void* a, const void* b, const float* sa,
+                                          const float* sb, const int32_t* problem_sizes,
+                                          const int32_t* expert_offsets, int num_experts, int total_rows, int n, int k,
+                                          int force_bm, void* stream) {
+  g_err[0] = 0;
+  int32_t* ws = nullptr;
+  size_t ws_bytes = 0;
+  int max_experts = 0;
+  int rc = esmoe_static_scratch(&ws, &ws_bytes, &max_experts);
+  if (rc) return fail(rc, "static workspace lookup failed: %s", hipGetErrorString((hipError_t)rc));
+  if (num_experts > max_experts)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "the static workspace holds the schedule of at most %d experts, got %d",
+                max_experts, num_experts);
+  return esmoe_fp8_blockwise_grouped_mm(out, out_dtype, a, b, sa, sb, problem_sizes, expert_offsets, num_experts,
+                                        total_rows, n, k, force_bm, ws, ws_bytes, stream);
 }
 
 int esmoe_fp8_blockwise_grouped_mm_swiglu_quant(void* q, float* scales, int mid_dtype, const void* a, const void* b,

@@ -40,6 +40,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "gemm_args.h"
 #include "mx_phase.h"
 #include "schedule.h"
@@ -878,6 +880,37 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
 }
 
 }  // namespace esmoe
+
+// Schedule workspace owned by the library, for callers that may not allocate (esmoe_fp8_blockwise_grouped_mm_static in
+// esmoe.h): room for the records and counters of kStaticScratchExperts experts.  Every GPU the library runs on holds
+// its own copy at its own address until the process ends; the name below is only the host-side handle of the
+// symbol, never a device address, so host code goes through esmoe_static_scratch().
+constexpr int kStaticScratchExperts = 1024;
+constexpr int kStaticScratchWords = (esmoe::kWsHeader + (kStaticScratchExperts + 1) * esmoe::kRecWords + 63) / 64 * 64;
+static __device__ __align__(256) int32_t scratch[kStaticScratchWords];
+
+// Device address and size of the current device's copy of the static workspace; the address is looked up once
+// per device (with that device current) and kept.
+extern "C" int esmoe_static_scratch(int32_t** ptr, size_t* bytes, int* max_experts) {
+  static int32_t* addr[64];
+  static std::mutex mu;
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return (int)err;
+  if (dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!addr[dev]) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return (int)err;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    addr[dev] = (int32_t*)p;
+  }
+  *ptr = addr[dev];
+  *bytes = sizeof(int32_t) * kStaticScratchWords;
+  *max_experts = kStaticScratchExperts;
+  return 0;
+}
 
 extern "C" int esmoe_launch_grouped_gemm(const esmoe::GemmArgs* args, int mx, int grid, hipStream_t stream) {
   using namespace esmoe;

@@ -63,6 +63,21 @@ int esmoe_fp8_blockwise_grouped_mm(void* out, int out_dtype, const void* a, cons
                                    size_t workspace_bytes, void* stream);
 
 /*
+ * esmoe_fp8_blockwise_grouped_mm for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc): same arguments without the workspace, same kernels, same
+ * results.  No counterpart in the reference, whose operator allocates its scratch tensors on every call
+ * (es_fp8_blockwise.cu:58-75).  The schedule workspace is a static array inside the library, one copy per GPU,
+ * ESMOE_STATIC_MAX_EXPERTS experts at most (more are rejected with ESMOE_ERR_INVALID_ARGUMENT); the call allocates
+ * and frees nothing.  All calls on one GPU share that array: calls that overlap in time on one GPU (two streams,
+ * two threads) race on it and must be serialised by the caller; calls ordered on one stream are safe.
+ */
+#define ESMOE_STATIC_MAX_EXPERTS 1024
+int esmoe_fp8_blockwise_grouped_mm_static(void* out, int out_dtype, const void* a, const void* b, const float* sa,
+                                          const float* sb, const int32_t* problem_sizes,
+                                          const int32_t* expert_offsets, int num_experts, int total_rows, int n, int k,
+                                          int force_bm, void* stream);
+
+/*
  * MXFP8 block-scaled grouped GEMM (e4m3 data, E8M0 scale per 1x32 block along K).
  * Replaces es_sm100_mxfp8_blockscaled_grouped_mm
  *   (expert_specialization/csrc/cuda/es_sm100_mxfp8_blockscaled.cu:5-40, schema
