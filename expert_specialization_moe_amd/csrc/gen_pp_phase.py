@@ -1,0 +1,185 @@
+"""Writes pp_phase.h: one K block of a tall fp8-blockwise tile as ONE inline-asm statement.
+
+    python gen_pp_phase.py > pp_phase.h
+
+The eight wavefronts of a tile form two groups of four (one wavefront of each group per SIMD); group 0 owns the upper
+half of the tile's token rows, group 1 the lower half, and every wavefront owns 64 of the 256 weight rows.  The groups
+run half a K block apart.  A K block of a wavefront is
+
+    memory phase   copies of coming stages global -> LDS, weight fragments and the first two token fragments
+                   LDS -> registers, the block's scales
+    s_barrier
+    matrix phase   MTW x 4 MFMAs; the fp32 promotion of MFMA j - 3 (four v_fmac) behind MFMA j; token fragment
+                   mt + 2 read from LDS behind the first MFMA of row tile mt (three fragment buffers)
+    s_barrier
+    the last three promotions (in the shadow of the other group's first MFMAs)
+
+so while one group's wavefront keeps its SIMD's matrix pipe busy, the other group's wavefront on that SIMD moves data.
+Written as a statement, not as C++ with scheduling fences: the compiler neither keeps such an order nor tracks the
+asynchronous copies (its own waits would land in the loop), and every register that lives only inside the K block
+(fragments, MFMA results, scales) is a fixed register named as a clobber, which leaves the compiler nothing to spill.
+
+Ring (see gemm_tile_pp): weight stages in 3 slots shared by both groups, token stages in 2 slots per group (each
+group copies and reads only its own token rows), activation scales in 3 chunk buffers of 4 K blocks per group.
+Copies issued in the memory phase of K block kb, oldest first:  one 16-row piece of scale chunk kb/4 + 2,  the
+group's token rows of K block kb + 1,  the wavefront's weight rows of K block kb + 2.  Waits (per wavefront, own copies):
+    end of the memory phase   vmcnt(nT + 5): everything older than this phase's copies, i.e. weights kb + 1
+    end of the matrix phase   vmcnt(4):      also the scale piece and the tokens of kb + 1; weights kb + 2 stay in flight
+Every barrier certifies to the other wavefronts what the waits before it completed.
+
+Hazards the assembler does not see (no hardware interlock between an MFMA's result and a vector-ALU read of it):
+a promotion follows its MFMA by three MFMAs and twelve v_fmac (at least 15 issue slots, 11 needed); the tail
+promotions follow the barrier; a fragment buffer is overwritten by a read that issues behind a later MFMA than
+the last one that used it, and LDS data returns much later than an MFMA reads its operands; s_nop 0 separates
+a write of m0 from the copy that uses it.
+"""
+import sys
+
+NT = 4
+ABLATE = set()   # timing experiments only (results wrong): "fma", "copy", "roll", "read", "barrier", "vmwait"
+
+
+def regs(lo, n):
+    return f"v[{lo}:{lo + n - 1}]"
+
+
+class Plan:
+    def __init__(self, mtw, fuse):
+        self.mtw, self.fuse = mtw, fuse
+        # fixed registers, from the top of the file down
+        self.w = [224 + 8 * n for n in range(4)]          # weight fragments
+        self.a = [200, 208, 216]                          # token fragment buffers
+        self.t = [184, 188, 192, 196]                     # MFMA results awaiting promotion
+        self.sa = (184 - (mtw + 2)) // 2 * 2              # sa[0..mtw-1] (sa * sb after the memory phase), sb, sb_up
+        self.sb = self.sa + mtw
+        self.sbu = self.sb + 1
+        self.scu = (self.sa - mtw) // 2 * 2 if fuse else None    # fused form: products sa * sb_up of the up half
+        self.lowest = self.scu if fuse else self.sa
+        self.ntc = mtw // 2                               # token copies per wavefront and K block
+
+    def clobbers(self):
+        return [f'"v{i}"' for i in range(self.lowest, 256)] + ['"memory"', '"m0"']
+
+
+def memory_phase(p):
+    L = []
+    rd = []   # LDS reads to interleave with the copies: (dst, addr, offset)
+    for n in range(4):
+        rd.append((regs(p.w[n], 4), "wl", n * 2048))
+        rd.append((regs(p.w[n] + 4, 4), "wh", n * 2048))
+    for mt in range(2):
+        rd.append((regs(p.a[mt], 4), "al", mt * 2048))
+        rd.append((regs(p.a[mt] + 4, 4), "ah", mt * 2048))
+    copies = [("s", None)] + [("t", i) for i in range(p.ntc)] + [("w", i) for i in range(4)]
+    per = (len(rd) + len(copies) - 1) // len(copies)
+    for kind, i in copies:
+        if kind == "s":
+            L += ["s_mov_b32 m0, %[ls]", "s_nop 0", "global_load_lds_dword %[vs], %[sp]"]
+        elif kind == "t":
+            if i == 0:
+                L += ["s_mov_b32 m0, %[la]", "s_nop 0"]
+            L.append(f"global_load_lds_dwordx4 %[va{i}], %[ap]" + (f" offset:{i * 1024}" if i else ""))
+        else:
+            if i == 0:
+                L += ["s_mov_b32 m0, %[lw]", "s_nop 0"]
+            L.append(f"global_load_lds_dwordx4 %[vw{i}], %[wp]" + (f" offset:{i * 1024}" if i else ""))
+        for _ in range(per):
+            if rd:
+                d, a, off = rd.pop(0)
+                L.append(f"ds_read_b128 {d}, %[{a}]" + (f" offset:{off}" if off else ""))
+    for d, a, off in rd:
+        L.append(f"ds_read_b128 {d}, %[{a}]" + (f" offset:{off}" if off else ""))
+    for mt in range(p.mtw):
+        L.append(f"ds_read_b32 v{p.sa + mt}, %[sal]" + (f" offset:{mt * 256}" if mt else ""))
+    L.append(f"ds_read_b32 v{p.sb}, %[sbl]")
+    if p.fuse:
+        L.append(f"ds_read_b32 v{p.sbu}, %[sbl] offset:1024")
+    L.append("s_waitcnt lgkmcnt(0)")
+    if p.fuse:
+        for mt in range(p.mtw):
+            L.append(f"v_mul_f32 v{p.scu + mt}, v{p.sa + mt}, v{p.sbu}")
+    for mt in range(p.mtw):
+        L.append(f"v_mul_f32 v{p.sa + mt}, v{p.sa + mt}, v{p.sb}")
+    L.append(f"s_waitcnt vmcnt({p.ntc + 5}) ; explicit")
+    L.append("s_barrier")
+    return L
+
+
+def promotion(p, j):
+    mt, nt = divmod(j, NT)
+    sc = p.scu + mt if (p.fuse and nt >= NT // 2) else p.sa + mt
+    return [f"v_fmac_f32 %[c{nt}_{mt}_{i}], v{p.t[j % 4] + i}, v{sc}" for i in range(4)]
+
+
+def matrix_phase(p):
+    L = []
+    total = p.mtw * NT
+    lag = 3
+    for j in range(total):
+        mt, nt = divmod(j, NT)
+        if nt == 0 and mt >= 2:
+            L.append("s_waitcnt lgkmcnt(2)" if mt + 1 < p.mtw else "s_waitcnt lgkmcnt(0)")
+        L.append(f"v_mfma_f32_16x16x128_f8f6f4 {regs(p.t[j % 4], 4)}, {regs(p.w[nt], 8)}, {regs(p.a[mt % 3], 8)}, 0")
+        if nt == 0 and mt + 2 < p.mtw:
+            b = p.a[(mt + 2) % 3]
+            L.append(f"ds_read_b128 {regs(b, 4)}, %[al] offset:{(mt + 2) * 2048}")
+            L.append(f"ds_read_b128 {regs(b + 4, 4)}, %[ah] offset:{(mt + 2) * 2048}")
+        if j >= lag:
+            L += promotion(p, j - lag)
+    L.append("s_waitcnt vmcnt(4) ; explicit")
+    L.append("s_barrier")
+    for j in range(total - lag, total):
+        L += promotion(p, j)
+    return L
+
+
+def ablated(lines):
+    out = []
+    for l in lines:
+        if "fma" in ABLATE and l.startswith("v_fmac"):
+            continue
+        if "halffma" in ABLATE and l.startswith("v_fmac") and l.split("]")[0][-1] in "13":
+            continue
+        if "copy" in ABLATE and l.startswith("global_load_lds"):
+            continue
+        if "read" in ABLATE and l.startswith("ds_read_b128") and "%[w" in l:
+            continue
+        if "roll" in ABLATE and l.startswith("ds_read_b128") and "%[a" in l and "offset" in l and int(l.split("offset:")[1]) >= 4096:
+            continue
+        if "barrier" in ABLATE and l == "s_barrier":
+            continue
+        if "vmwait" in ABLATE and l.startswith("s_waitcnt vmcnt"):
+            continue
+        out.append(l)
+    return out
+
+
+def emit(name, mtw, fuse):
+    p = Plan(mtw, fuse)
+    lines = ablated(memory_phase(p) + matrix_phase(p))
+    print(f"#define {name}_BODY \\")
+    for i, l in enumerate(lines):
+        last = i + 1 == len(lines)
+        print('  "%s%s"%s' % (l, "" if last else "\\n\\t", "" if last else " \\"))
+    print(f"#define {name}_OUTS " + ", ".join(
+        f'[c{nt}_{mt}_{i}] "+v"(acc[{nt}][{mt}][{i}])' for mt in range(mtw) for nt in range(NT) for i in range(4)))
+    ins = [f'[va{i}] "v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "v"(vw[{i}])' for i in range(4)]
+    ins += ['[vs] "v"(vsq)', '[wl] "v"(wl)', '[wh] "v"(wh)', '[al] "v"(al)', '[ah] "v"(ah)', '[sal] "v"(sal)', '[sbl] "v"(sbl)',
+            '[la] "s"(la)', '[lw] "s"(lw)', '[ls] "s"(ls)', '[ap] "s"(ap)', '[wp] "s"(wp)', '[sp] "s"(sp)']
+    print(f"#define {name}_INS " + ", ".join(ins))
+    print(f"#define {name}_CLOBBERS " + ", ".join(p.clobbers()))
+    print(f"#define {name}_LOWEST_FIXED_VGPR {p.lowest}")
+
+
+def main():
+    for a in sys.argv[1:]:
+        ABLATE.add(a)
+    print("// Generated by gen_pp_phase.py; do not edit.")
+    print("#pragma once")
+    for mtw in (4, 6):
+        emit(f"ESMOE_PP{mtw * 2}", mtw, False)
+        emit(f"ESMOE_PP{mtw * 2}F", mtw, True)
+
+
+if __name__ == "__main__":
+    main()

@@ -44,6 +44,11 @@
 
 #include "gemm_args.h"
 #include "mx_phase.h"
+#ifdef ESMOE_PP_HEADER
+#include ESMOE_PP_HEADER
+#else
+#include "pp_phase.h"
+#endif
 #include "schedule.h"
 #include "swiglu.h"
 
@@ -157,6 +162,99 @@ struct TileGeom {
   static constexpr int kCopiesPerStage = kACopies + kWCopies + 1;       // + 1 scale copy
   static_assert(kNBuf >= 2, "ring too small");
 };
+
+// Epilogue of a tile: `acc[nt][mt][i]` holds, for this lane, columns n0 + nw + nt*16 + 4*gq + i of token row
+// m0 + mw + mt*16 + r (gq = lane / 16, r = lane % 16).  Plain form: convert and store.  FUSE: SwiGLU and the 1x128
+// quantisation (the wavefront's first NTW/2 column tiles are gate columns, the rest the matching up columns).
+// `lds` is scratch for the fused form and must be free: every wavefront has left the K loop.
+template <int BM, int MTW, int NTW, int kWavesN, bool FUSE, typename Acc>
+__device__ __forceinline__ void tile_epilogue(const GemmArgs& g, Acc& acc, int M, int m0, int n0, long row_base, int mw,
+                                              int nw, int wn, int lane, bool wave_active, uint8_t* lds) {
+  const int r = lane & 15, gq = lane >> 4;
+  const int N = g.n;
+  if constexpr (FUSE) {
+    // Lane holds, of token row mw + mt*16 + r, gate (n-tiles 0 .. NTW/2-1) and up (the other half) of the h columns
+    // wn*RW/2 + nt*16 + 4*gq + [0,4) of the tile's 128.  Same arithmetic, in the same order, as the unfused
+    // sequence: projection rounded to the output type, silu(gate) * up in fp32, rounded to the output type, then
+    // the 1x128 quantisation (block maximum floored at 1e-4, multiplier (1/amax)*448, scale amax*(1/448)).
+    constexpr int kHalf = NTW / 2, kRW = NTW * 16;
+    const bool f16 = g.out_dtype != 0;
+    float* s_amax = (float*)lds;   // [kWavesN][BM]; the ring is free: every wavefront has left the K loop
+    float h[MTW][kHalf][4];
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) {
+      float amax = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < kHalf; nt++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float gv, uv;
+          if (f16) {
+            gv = (float)(_Float16)acc[nt][mt][i];
+            uv = (float)(_Float16)acc[nt + kHalf][mt][i];
+          } else {
+            gv = (float)(__bf16)acc[nt][mt][i];
+            uv = (float)(__bf16)acc[nt + kHalf][mt][i];
+          }
+          float hv = swiglu_f32(gv, uv);
+          hv = f16 ? (float)(_Float16)hv : (float)(__bf16)hv;
+          h[mt][nt][i] = hv;
+          amax = __builtin_fmaxf(amax, __builtin_fabsf(hv));
+        }
+      }
+      amax = __builtin_fmaxf(amax, __shfl_xor(amax, 16));
+      amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32));
+      if (gq == 0) s_amax[wn * BM + mw + mt * 16 + r] = amax;
+    }
+    __syncthreads();
+    const int inter = N >> 1;
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) {
+      const int row = mw + mt * 16 + r;
+      float amax = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWavesN; w++) amax = __builtin_fmaxf(amax, s_amax[w * BM + row]);
+      amax = __builtin_fmaxf(amax, 1e-4f);
+      const float mult = (1.0f / amax) * 448.0f;
+      const int m = m0 + row;
+      if (m < M) {
+        uint8_t* qrow = (uint8_t*)g.q_out + (row_base + m) * (long)inter + (n0 >> 1) + wn * (kRW / 2) + gq * 4;
+#pragma unroll
+        for (int nt = 0; nt < kHalf; nt++) {
+          float y[4];
+#pragma unroll
+          for (int i = 0; i < 4; i++) y[i] = __builtin_amdgcn_fmed3f(h[mt][nt][i] * mult, -448.f, 448.f);
+          int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+          w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+          *(int*)(qrow + nt * 16) = w0;
+        }
+        if (gq == 0 && wn == 0) g.scales_out[(row_base + m) * (long)(inter >> 7) + (n0 >> 8)] = amax * (1.0f / 448.0f);
+      }
+    }
+    __syncthreads();   // s_amax is ring memory: the next tile's copies must not land before every lane has read it
+    return;
+  }
+  // epilogue: lane holds columns n0 + nw + nt*16 + 4*gq + [0,4) of token row m0 + mw + mt*16 + r
+  if (wave_active) {
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) {
+      int m = m0 + mw + mt * 16 + r;
+      if (m < M) {
+        long orow = (row_base + m) * (long)N;
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) {
+          int n = n0 + nw + nt * 16 + gq * 4;
+          const v4f v = {acc[nt][mt][0], acc[nt][mt][1], acc[nt][mt][2], acc[nt][mt][3]};
+          if (g.out_dtype == 0) {
+            *(bf16x4*)((__bf16*)g.out + orow + n) = __builtin_convertvector(v, bf16x4);
+          } else {
+            *(f16x4*)((_Float16*)g.out + orow + n) = __builtin_convertvector(v, f16x4);
+          }
+        }
+      }
+    }
+  }
+}
 
 // FUSE (fp8-blockwise only): the weights are a gate_up projection [E, 2I, K] (gate rows first) and the tile's 256
 // weight rows are 128 gate rows and the matching 128 up rows, interleaved so that every wavefront holds gate and up
@@ -636,87 +734,170 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   }
   if (kPP && grp == 0) block_barrier();
 
-  if constexpr (FUSE) {
-    // Lane holds, of token row mw + mt*16 + r, gate (n-tiles 0 .. NTW/2-1) and up (the other half) of the h columns
-    // wn*RW/2 + nt*16 + 4*gq + [0,4) of the tile's 128.  Same arithmetic, in the same order, as the unfused
-    // sequence: projection rounded to the output type, silu(gate) * up in fp32, rounded to the output type, then
-    // the 1x128 quantisation (block maximum floored at 1e-4, multiplier (1/amax)*448, scale amax*(1/448)).
-    constexpr int kHalf = NTW / 2, kRW = NTW * 16;
-    const bool f16 = g.out_dtype != 0;
-    float* s_amax = (float*)lds;   // [kWavesN][BM]; the ring is free: every wavefront has left the K loop
-    float h[MTW][kHalf][4];
+  tile_epilogue<G::BM, MTW, NTW, G::kWavesN, FUSE>(g, acc, M, m0, n0, row_base, mw, nw, wn, lane, wave_active, lds);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tall fp8-blockwise tiles (MT = 8 or 12, K a multiple of 512): the K block is one hand-scheduled statement
+// (pp_phase.h, written by gen_pp_phase.py) and the ring is split by operand.
+//
+//   LDS   [0, 96 KB)            weight stages, 3 slots of 256 rows x 128 B, shared by the two groups
+//         then 4 token regions  group g (wavefronts 4g .. 4g+3, token rows g*GR .. +GR of the tile), 2 slots each:
+//                               a group copies, reads and refills only its own rows, so its refill waits for nobody else
+//         then 6 scale chunks   sa of the group's rows for 4 K blocks (16 B per row), 3 buffers per group, fetched
+//                               two chunks ahead in 16-row pieces, one piece per wavefront and K block
+//         then the weight block scales of the tile, [2 column blocks][K blocks]
+//
+// Timeline in half K blocks h (barrier intervals): group 0 runs the memory phase of K block kb in h = 2kb and its matrix
+// phase in 2kb + 1, group 1 one interval later.  Weight stage kb is read in 2kb and 2kb + 1 (memory phases only) and its
+// slot is refilled with stage kb + 3 from 2kb + 2 on, three or more intervals before 2kb + 6; a group's token stage
+// kb is read in its memory and matrix phase of kb and refilled in its memory phase of kb + 1 with stage kb + 2.
+template <int MT, bool FUSE>
+__device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds,
+                                             uint32_t* timeline = nullptr) {
+  static_assert(MT == 8 || MT == 12, "hand-scheduled K block: 128- and 192-row tiles");
+  constexpr int MTW = MT / 2, NTW = 4, BM = MT * 16, GR = MTW * 16;
+  constexpr int kTCopies = MTW / 2;                 // token copies per wavefront and K block (8 rows each)
+  constexpr int kWSlot = kBN * 128, kTSlot = GR * 128, kSaBuf = 128 * 16;
+  constexpr int kTBase = 3 * kWSlot, kSaBase = kTBase + 4 * kTSlot, kSbBase = kSaBase + 6 * kSaBuf;
+  static_assert(kSbBase + 2 * kMaxKB * 4 <= kLdsBytes, "LDS map of the split ring");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2, wj = wave & 3;
+  const int r = lane & 15, gq = lane >> 4;
+  const int K = g.k, N = g.n, KB = K >> 7, NCH = KB >> 2;
+  const long row_base = g.expert_offsets[e];
+  const int nw = wj * 64, mw = grp * GR;
+  const bool wave_active = n0 + nw < N;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+
+  // ---- copy plan (see gemm_tile for the slot permutation and the instruction offsets) ----------------------
+  constexpr int kBias = 3072;
+  const int crow = lane >> 3, cslot = lane & 7;
+  const int a_last = M - 1 - m0;
+  uint32_t va[kTCopies], vw[4], vs[4];
 #pragma unroll
-    for (int mt = 0; mt < MTW; mt++) {
-      float amax = 0.f;
-#pragma unroll
-      for (int nt = 0; nt < kHalf; nt++) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          float gv, uv;
-          if (f16) {
-            gv = (float)(_Float16)acc[nt][mt][i];
-            uv = (float)(_Float16)acc[nt + kHalf][mt][i];
-          } else {
-            gv = (float)(__bf16)acc[nt][mt][i];
-            uv = (float)(__bf16)acc[nt + kHalf][mt][i];
-          }
-          float hv = swiglu_f32(gv, uv);
-          hv = f16 ? (float)(_Float16)hv : (float)(__bf16)hv;
-          h[mt][nt][i] = hv;
-          amax = __builtin_fmaxf(amax, __builtin_fabsf(hv));
-        }
-      }
-      amax = __builtin_fmaxf(amax, __shfl_xor(amax, 16));
-      amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32));
-      if (gq == 0) s_amax[wn * G::BM + mw + mt * 16 + r] = amax;
-    }
-    __syncthreads();
-    const int inter = N >> 1;
-#pragma unroll
-    for (int mt = 0; mt < MTW; mt++) {
-      const int row = mw + mt * 16 + r;
-      float amax = 0.f;
-#pragma unroll
-      for (int w = 0; w < G::kWavesN; w++) amax = __builtin_fmaxf(amax, s_amax[w * G::BM + row]);
-      amax = __builtin_fmaxf(amax, 1e-4f);
-      const float mult = (1.0f / amax) * 448.0f;
-      const int m = m0 + row;
-      if (m < M) {
-        uint8_t* qrow = (uint8_t*)g.q_out + (row_base + m) * (long)inter + (n0 >> 1) + wn * (kRW / 2) + gq * 4;
-#pragma unroll
-        for (int nt = 0; nt < kHalf; nt++) {
-          float y[4];
-#pragma unroll
-          for (int i = 0; i < 4; i++) y[i] = __builtin_amdgcn_fmed3f(h[mt][nt][i] * mult, -448.f, 448.f);
-          int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
-          w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
-          *(int*)(qrow + nt * 16) = w0;
-        }
-        if (gq == 0 && wn == 0) g.scales_out[(row_base + m) * (long)(inter >> 7) + (n0 >> 8)] = amax * (1.0f / 448.0f);
-      }
-    }
-    __syncthreads();   // s_amax is ring memory: the next tile's copies must not land before every lane has read it
-    return;
+  for (int i = 0; i < kTCopies; i++) {
+    const int lrow = (wj * kTCopies + i) * 8 + crow;      // row inside the group's token region
+    const int trow = mw + lrow;
+    const int grow = trow > a_last ? a_last : trow;
+    va[i] = (uint32_t)grow * (uint32_t)K + (swz(lrow, cslot) << 4) + kBias - i * 1024;
   }
-  // epilogue: lane holds columns n0 + nw + nt*16 + 4*gq + [0,4) of token row m0 + mw + mt*16 + r
-  if (wave_active) {
 #pragma unroll
-    for (int mt = 0; mt < MTW; mt++) {
-      int m = m0 + mw + mt * 16 + r;
-      if (m < M) {
-        long orow = (row_base + m) * (long)N;
+  for (int i = 0; i < 4; i++) {
+    const int blk = wave * 4 + i;
+    int row;
+    if constexpr (FUSE) {
+      constexpr int kRW = NTW * 16, kBlocks = kRW / 8, kHalfBlocks = kBlocks / 2;
+      const int wcol = blk / kBlocks, within = blk % kBlocks;
+      row = (within / kHalfBlocks) * (N >> 1) + (n0 >> 1) + wcol * (kRW / 2) + (within % kHalfBlocks) * 8;
+    } else {
+      row = (n0 + blk * 8 < N ? blk : i) * 8;
+    }
+    vw[i] = (uint32_t)(row + crow) * (uint32_t)K + (swz(blk * 8 + crow, cslot) << 4) + kBias - i * 1024;
+  }
+  // scale pieces: in K block kb (q = kb % 4) wavefront wj fetches rows (wj & 1)*64 + q*16 .. +16 of a chunk, lane ->
+  // (row lane / 4, K block lane % 4 of the chunk); wavefronts 2 and 3 repeat what 0 and 1 fetch
 #pragma unroll
-        for (int nt = 0; nt < NTW; nt++) {
-          int n = n0 + nw + nt * 16 + gq * 4;
-          if (g.out_dtype == 0) {
-            *(bf16x4*)((__bf16*)g.out + orow + n) = __builtin_convertvector(acc[nt][mt], bf16x4);
-          } else {
-            *(f16x4*)((_Float16*)g.out + orow + n) = __builtin_convertvector(acc[nt][mt], f16x4);
-          }
-        }
-      }
+  for (int q = 0; q < 4; q++) {
+    const int trow = mw + (wj & 1) * 64 + q * 16 + (lane >> 2);
+    const int grow = trow > a_last ? a_last : trow;
+    vs[q] = (uint32_t)grow * (uint32_t)KB * 4 + (lane & 3) * 4;
+  }
+  const uint8_t* a_ptr = (const uint8_t*)g.a + (row_base + m0) * K - kBias;
+  const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + (FUSE ? 0 : n0)) * K - kBias;
+  const uint8_t* sa_ptr = (const uint8_t*)(g.sa + (row_base + m0) * KB);
+  const uint32_t t_dst = lds0 + kTBase + grp * 2 * kTSlot + wj * kTCopies * 1024;   // + slot * kTSlot
+  const uint32_t w_dst = lds0 + wave * 4096;                                        // + slot * kWSlot
+  const uint32_t s_dst = lds0 + kSaBase + grp * 3 * kSaBuf + (wj & 1) * 64 * 16;    // + buffer * kSaBuf + q * 256
+  auto issue_t = [&](int kb, int slot) { dma16xn<false>(t_dst + slot * kTSlot, a_ptr + (long)kb * 128, va); };
+  auto issue_w = [&](int kb, int slot) { dma16xn<false>(w_dst + slot * kWSlot, w_ptr + (long)kb * 128, vw); };
+
+  // ---- fragment and scale read plan --------------------------------------------------------------------------
+  const uint32_t wfrag = lds0 + (nw + r) * 128 + swz(r, gq) * 16;                       // + slot * kWSlot, n-tile nt at + nt*2048
+  const uint32_t afrag = lds0 + kTBase + grp * 2 * kTSlot + r * 128 + swz(r, gq) * 16;  // + slot * kTSlot, row tile mt at + mt*2048
+  const uint32_t sa_rd = lds0 + kSaBase + grp * 3 * kSaBuf + r * 16;                    // + buffer * kSaBuf + q*4, row tile mt at + mt*256
+  const uint32_t sb_rd = lds0 + kSbBase + (FUSE ? 0 : (nw >> 7)) * kMaxKB * 4;          // + kb*4 (FUSE: up block at + kMaxKB*4)
+
+  float acc[NTW][MTW][4];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) acc[nt][mt][i] = 0.f;
+
+  // ---- prologue: weight block scales of the tile, scale chunks 0 and 1, token stage 0, weight stages 0 and 1 ----
+  {
+    const int blk = wave >> 2, kb0 = (wave & 3) * 64;
+    if (kb0 < KB) {
+      int nb = (n0 >> 7) + blk;
+      if (nb * 128 >= N) nb = n0 >> 7;
+      if constexpr (FUSE) nb = (n0 >> 8) + blk * (N >> 8);
+      const int kbi = kb0 + lane < KB ? kb0 + lane : KB - 1;
+      dma4(g.sb + ((long)e * (N >> 7) + nb) * KB, (uint32_t)kbi * 4, lds0 + kSbBase + (blk * kMaxKB + kb0) * 4);
     }
   }
+  {
+    // chunk (wj >> 1), rows (wj & 1)*64 + lane of the group: 16 bytes per row
+    const int ch = (wj >> 1) < NCH ? (wj >> 1) : NCH - 1;
+    const int trow = mw + (wj & 1) * 64 + lane;
+    const int grow = trow > a_last ? a_last : trow;
+    dma16(sa_ptr + (long)ch * 16, (uint32_t)grow * (uint32_t)KB * 4, lds0 + kSaBase + (grp * 3 + (wj >> 1)) * kSaBuf + (wj & 1) * 1024);
+  }
+  issue_t(0, 0);
+  issue_w(0, 0);
+  issue_w(1 < KB ? 1 : KB - 1, 1);
+  wait_vmcnt<4>();
+  block_barrier();
+  if (grp == 1) block_barrier();
+
+#ifdef ESMOE_TIMELINE
+  const uint64_t tl_r0 = __builtin_amdgcn_s_memrealtime(), tl_c0 = __builtin_amdgcn_s_memtime();
+#endif
+  int tslot = 0, wslot = 0, sabuf = 0;   // slots of K block kb: tokens kb % 2, weights kb % 3, scale chunk (kb / 4) % 3
+  for (int kb = 0; kb < KB; kb++) {
+    const int q = kb & 3;
+    const int kbt = kb + 1 < KB ? kb + 1 : KB - 1, kbw = kb + 2 < KB ? kb + 2 : KB - 1;
+    const int chw = (kb >> 2) + 2 < NCH ? (kb >> 2) + 2 : NCH - 1;
+    const int wnext = wslot >= 1 ? wslot - 1 : 2;          // (kb + 2) % 3
+    const int sanext = sabuf >= 1 ? sabuf - 1 : 2;         // (kb / 4 + 2) % 3
+    const uint32_t la = t_dst + (tslot ^ 1) * kTSlot, lw = w_dst + wnext * kWSlot;
+    const uint32_t ls = s_dst + sanext * kSaBuf + q * 256;
+    const uint8_t* ap = a_ptr + (long)kbt * 128;
+    const uint8_t* wp = w_ptr + (long)kbw * 128;
+    const uint8_t* sp = sa_ptr + (long)chw * 16;
+    const uint32_t wl = wfrag + wslot * kWSlot, wh = wl ^ 64;
+    const uint32_t al = afrag + tslot * kTSlot, ah = al ^ 64;
+    const uint32_t sal = sa_rd + sabuf * kSaBuf + q * 4;
+    const uint32_t sbl = sb_rd + kb * 4;
+    const uint32_t vsq = vs[0];
+    if constexpr (MT == 12) {
+      if constexpr (FUSE) asm volatile(ESMOE_PP12F_BODY : ESMOE_PP12F_OUTS : ESMOE_PP12F_INS : ESMOE_PP12F_CLOBBERS);
+      else asm volatile(ESMOE_PP12_BODY : ESMOE_PP12_OUTS : ESMOE_PP12_INS : ESMOE_PP12_CLOBBERS);
+    } else {
+      if constexpr (FUSE) asm volatile(ESMOE_PP8F_BODY : ESMOE_PP8F_OUTS : ESMOE_PP8F_INS : ESMOE_PP8F_CLOBBERS);
+      else asm volatile(ESMOE_PP8_BODY : ESMOE_PP8_OUTS : ESMOE_PP8_INS : ESMOE_PP8_CLOBBERS);
+    }
+    // the piece offsets rotate with q; slots advance
+    { const uint32_t t = vs[0]; vs[0] = vs[1]; vs[1] = vs[2]; vs[2] = vs[3]; vs[3] = t; }
+    tslot ^= 1;
+    wslot = wslot == 2 ? 0 : wslot + 1;
+    if (q == 3) sabuf = sabuf == 2 ? 0 : sabuf + 1;
+  }
+#ifdef ESMOE_TIMELINE
+  if (timeline && tid == 0) {   // debug build: K loop start and end (100 MHz ticks), its length in shader clocks
+    timeline[4] = (uint32_t)tl_r0;
+    timeline[5] = (uint32_t)__builtin_amdgcn_s_memrealtime();
+    timeline[6] = (uint32_t)(__builtin_amdgcn_s_memtime() - tl_c0);
+  }
+#endif
+  // the copies past the last K block (they fetched it again) must have landed before anything reuses the ring
+  wait_vmcnt<0>();
+  if (grp == 0) block_barrier();
+  block_barrier();
+  tile_epilogue<BM, MTW, NTW, 4, FUSE>(g, acc, M, m0, n0, row_base, mw, nw, wj, lane, wave_active, lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -784,6 +965,10 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
   if (num_experts < kXcds && e >= num_experts && e < kXcds) ws[kWsXcdCounter + e] = 0;
 }
 
+// Heights whose fp8-blockwise tiles run the hand-scheduled K block of gemm_tile_pp (bit 0: 128 rows, bit 1: 192 rows).
+#ifndef ESMOE_PP_HEIGHTS
+#define ESMOE_PP_HEIGHTS 3
+#endif
 // Tile heights (MT * 16 rows) compiled into the persistent kernel.
 #ifndef ESMOE_VARIANTS
 #define ESMOE_VARIANTS ESMOE_CASE(1) ESMOE_CASE(2) ESMOE_CASE(4) ESMOE_CASE(8) ESMOE_CASE(12) ESMOE_CASE(16)
@@ -791,8 +976,9 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 
 template <bool MX, bool FUSE>
 __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
   __shared__ int s_item;
+  __shared__ int s_counters[kXcds + 1];
   int* ws = g.ws;
   const int hblocks = ws[kWsHeavyBlocks];
   const int ltotal = ws[kWsLightTotal];
@@ -806,6 +992,13 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   const int per_xcd = (int)gridDim.x / kXcds > 0 ? (int)gridDim.x / kXcds : 1;
   const bool light_first = (int)(blockIdx.x / kXcds) * 32 / per_xcd >= 32 - ws[kWsLightShare];
   int phase = 0, q = 0;
+  // Queues known to be exhausted (bits 0-7: the XCDs' heavy queues, bit 8: the light items).  When a draw comes back
+  // past the end of its queue, one look at all nine counters marks every queue that has run dry, so that a workgroup
+  // leaving its own queue does not spend an atomic round trip (about a microsecond under load) on each empty one.
+  int dead = ltotal == 0 ? 256 : 0;
+#pragma unroll
+  for (int x = 0; x < kXcds; x++)
+    if (x >= hblocks) dead |= 1 << x;
 #ifdef ESMOE_TIMELINE
   int tl_n = 0;
   if (threadIdx.x == 0) ((uint32_t*)ws)[4096 + blockIdx.x * 256] = 0;
@@ -813,7 +1006,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   for (;;) {
     const bool light = (phase == 0) == light_first;
     const int xq = (xcd + q) & (kXcds - 1);
-    if (light ? ltotal == 0 : xq >= hblocks) {   // nothing of this kind (or this queue never had a block)
+    if ((dead >> (light ? 8 : xq)) & 1) {   // nothing (left) in this queue: the next XCD's, then the other kind
       if (light || ++q == kXcds) {
         q = 0;
         if (++phase == 2) break;
@@ -831,12 +1024,20 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
 #else
     const int v = light ? ticket : sched_ticket_block(xq, ticket);
 #endif
-    if (v >= (light ? ltotal : hblocks)) {   // this queue is exhausted: the next XCD's, then the other kind
-      __syncthreads();                        // s_item is rewritten next
-      if (light || ++q == kXcds) {
-        q = 0;
-        if (++phase == 2) break;
+    if (v >= (light ? ltotal : hblocks)) {   // this queue is exhausted: see which others are
+      dead |= 1 << (light ? 8 : xq);
+      __syncthreads();                        // s_item and s_counters are rewritten next
+      if (threadIdx.x < kXcds + 1)
+        s_counters[threadIdx.x] = __hip_atomic_load(threadIdx.x < kXcds ? &ws[kWsXcdCounter + threadIdx.x] : &ws[kWsLightCounter],
+                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+#pragma unroll
+      for (int x = 0; x < kXcds; x++) {
+        // queue x holds the blocks x, x + 8, ...: 32 tickets each
+        const int tickets = x < hblocks ? ((hblocks - x + kXcds - 1) / kXcds) * kBlkTiles : 0;
+        if (__builtin_amdgcn_readfirstlane(s_counters[x]) >= tickets) dead |= 1 << x;
       }
+      if (__builtin_amdgcn_readfirstlane(s_counters[kXcds]) >= ltotal) dead |= 256;
       continue;
     }
     // schedule position of v: the last one whose first block (item) is <= v, found by bisection over the prefix
@@ -858,10 +1059,28 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     }
 #ifdef ESMOE_TIMELINE
     const uint64_t tl_t0 = __builtin_amdgcn_s_memrealtime();
+#define ESMOE_TL_PTR (tl_n < 31 ? (uint32_t*)ws + 4096 + blockIdx.x * 256 + 8 + tl_n * 8 : nullptr)
+#else
+#define ESMOE_TL_PTR nullptr
 #endif
-    switch (t.mt) {
-      ESMOE_VARIANTS
-      default: break;
+    // tall fp8-blockwise tiles take the hand-scheduled K block when the scale chunks fit K (a multiple of 512)
+    bool hand_scheduled = false;
+    if constexpr (!MX) {
+      if ((g.k & 511) == 0) {
+        if ((ESMOE_PP_HEIGHTS & 2) && t.mt == 12) {
+          gemm_tile_pp<12, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+          hand_scheduled = true;
+        } else if ((ESMOE_PP_HEIGHTS & 1) && t.mt == 8) {
+          gemm_tile_pp<8, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+          hand_scheduled = true;
+        }
+      }
+    }
+    if (!hand_scheduled) {
+      switch (t.mt) {
+        ESMOE_VARIANTS
+        default: break;
+      }
     }
 #ifdef ESMOE_TIMELINE
     // debug build only: (start, end, kind, position) of this workgroup's first 31 tiles, in 100 MHz ticks, 8 words

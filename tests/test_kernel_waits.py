@@ -28,7 +28,13 @@ def _build_module():
 def _mfma_loops(asm_text):
     """{(function, loop header, depth): [(line number, instruction)]} for inner loops that contain MFMAs."""
     func, hdr, blocks = None, None, {}
-    for i, line in enumerate(asm_text.split("\n")):
+    lines_all = asm_text.split("\n")
+    for i, line in enumerate(lines_all):
+        if re.match(r"^\.LBB\d+_\d+:", line):   # the loop comment of a block may continue on the following lines
+            j = i + 1
+            while j < len(lines_all) and lines_all[j].lstrip().startswith(";"):
+                line += " " + lines_all[j].strip()
+                j += 1
         m = re.match(r"^(_ZN5esmoe\w+):", line)
         if m:
             func, hdr = m.group(1), None
