@@ -80,7 +80,7 @@ int current_device_info(DeviceInfo* out) {
 // ESMOE_* environment variables (tuning aids) are read once per process, on the first GEMM launch; a value the
 // kernels cannot honour is reported by every launch instead of being applied.
 struct Knobs {
-  int big_mt_fp8 = 12, big_mt_mx = 16, order = 0, light_share = -1, wgs_per_cu = 1;
+  int big_mt_fp8 = 12, big_mt_mx = 12, order = 0, light_share = -1, wgs_per_cu = 1;
   char error[160] = "";
 };
 
@@ -94,11 +94,8 @@ const Knobs& knobs() {
     const char* big = getenv("ESMOE_BIG_MT");
     if (big && *big) {
       const int v = atoi(big);
-      // mxfp8 tiles of 128 and 256 rows read their token scales assuming a start on a 128-row boundary, which
-      // full tiles of 192 rows would break for the remainder tile: 8 and 16 only.
-      if (v == 8 || v == 16) r.big_mt_fp8 = r.big_mt_mx = v;
-      else if (v == 12) r.big_mt_fp8 = v;
-      else snprintf(r.error, sizeof(r.error), "ESMOE_BIG_MT=%s: full tiles are 8, 12 or 16 x 16 rows (8 or 16 for mxfp8)", big);
+      if (v == 8 || v == 12 || v == 16) r.big_mt_fp8 = r.big_mt_mx = v;
+      else snprintf(r.error, sizeof(r.error), "ESMOE_BIG_MT=%s: full tiles are 8, 12 or 16 x 16 rows", big);
     }
     r.order = env_int("ESMOE_ORDER", 0);
     if (r.order < 0 || r.order > 2) snprintf(r.error, sizeof(r.error), "ESMOE_ORDER must be 0, 1 or 2");
@@ -115,10 +112,11 @@ const Knobs& knobs() {
 esmoe::SchedPolicy default_policy(int force_bm, int mx) {
   esmoe::SchedPolicy p;
   p.force_mt = force_bm / 16;
-  // Taller tiles do more MFMA work per byte copied into LDS.  The mxfp8 kernel is fastest with 256-row
-  // tiles; the fp8-blockwise kernel, whose fp32 promotion shares the vector ALU, gains nothing beyond
-  // 192 rows, and shorter full tiles leave less padding in the remainder tile.
-  p.big_mt = mx ? 16 : 12;
+  // Full tiles are 192 rows for both kernels: the tallest tile whose ring (three weight stages, two token stages per
+  // wavefront group) fits the 160 KB of LDS, which is what the hand-scheduled K block of the tall tiles needs; 256-row
+  // tiles do more MFMA work per byte copied but run with a two-stage ring and measured slower.
+  (void)mx;
+  p.big_mt = 12;
   p.order = 0;
   p.light_share = -1;
   return p;

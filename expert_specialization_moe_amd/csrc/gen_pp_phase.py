@@ -133,6 +133,17 @@ def matrix_phase(p):
     return L
 
 
+def print_body(name, lines):
+    """The statement, and its form for weight rows that no other tile reads (non-temporal hint on the weight copies)."""
+    for suffix, hint in (("", ""), ("_NT", " nt")):
+        print(f"#define {name}_BODY{suffix} \\")
+        for i, l in enumerate(lines):
+            last = i + 1 == len(lines)
+            if l.startswith("global_load_lds_dwordx4 %[vw"):
+                l += hint
+            print('  "%s%s"%s' % (l, "" if last else "\\n\\t", "" if last else " \\"))
+
+
 def ablated(lines):
     out = []
     for l in lines:
@@ -157,15 +168,106 @@ def ablated(lines):
 def emit(name, mtw, fuse):
     p = Plan(mtw, fuse)
     lines = ablated(memory_phase(p) + matrix_phase(p))
-    print(f"#define {name}_BODY \\")
-    for i, l in enumerate(lines):
-        last = i + 1 == len(lines)
-        print('  "%s%s"%s' % (l, "" if last else "\\n\\t", "" if last else " \\"))
+    print_body(name, lines)
     print(f"#define {name}_OUTS " + ", ".join(
         f'[c{nt}_{mt}_{i}] "+v"(acc[{nt}][{mt}][{i}])' for mt in range(mtw) for nt in range(NT) for i in range(4)))
     ins = [f'[va{i}] "v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "v"(vw[{i}])' for i in range(4)]
     ins += ['[vs] "v"(vsq)', '[wl] "v"(wl)', '[wh] "v"(wh)', '[al] "v"(al)', '[ah] "v"(ah)', '[sal] "v"(sal)', '[sbl] "v"(sbl)',
             '[la] "s"(la)', '[lw] "s"(lw)', '[ls] "s"(ls)', '[ap] "s"(ap)', '[wp] "s"(wp)', '[sp] "s"(sp)']
+    print(f"#define {name}_INS " + ", ".join(ins))
+    print(f"#define {name}_CLOBBERS " + ", ".join(p.clobbers()))
+    print(f"#define {name}_LOWEST_FIXED_VGPR {p.lowest}")
+
+
+# ---- mxfp8 form ----------------------------------------------------------------------------------------------------
+# Same ring and phases with the hardware-scaled MFMA accumulating straight into the accumulators: no promotions, no
+# result buffers.  The E8M0 scale bytes travel with the stages as verbatim 512-byte scale tiles (2 for the weight
+# rows behind a weight stage, 2 for the group's token rows behind its token stage); every wavefront issues one
+# 1 KB scale copy per K block so that the counted waits are the same for all (wavefront 0: weight scales of K block
+# kb + 2, wavefronts 1 and 5: their group's token scales of kb + 1, the others re-read one line into a spare area).
+# A lane reads the scale dword of its row and shifts its K sub-block's byte (lane / 16) down to byte 0.
+class MxPlan:
+    def __init__(self, mtw):
+        self.mtw = mtw
+        self.w = [224 + 8 * n for n in range(4)]
+        self.a = [200, 208, 216]
+        self.sfw = 196                      # 4 weight-row scale registers
+        self.sfa = 196 - mtw - (mtw % 2)    # mtw token-row scale registers
+        self.lowest = self.sfa
+        self.ntc = mtw // 2
+
+    def clobbers(self):
+        return [f'"v{i}"' for i in range(self.lowest, 256)] + ['"memory"', '"m0"']
+
+
+def mx_memory_phase(p):
+    L, rd = [], []
+    for n in range(4):
+        rd.append((regs(p.w[n], 4), "wl", n * 2048))
+        rd.append((regs(p.w[n] + 4, 4), "wh", n * 2048))
+    for mt in range(2):
+        rd.append((regs(p.a[mt], 4), "al", mt * 2048))
+        rd.append((regs(p.a[mt] + 4, 4), "ah", mt * 2048))
+    copies = [("s", None)] + [("t", i) for i in range(p.ntc)] + [("w", i) for i in range(4)]
+    per = (len(rd) + len(copies) - 1) // len(copies)
+    for kind, i in copies:
+        if kind == "s":
+            L += ["s_mov_b32 m0, %[ls]", "s_nop 0", "global_load_lds_dwordx4 %[vs], %[sp]"]
+        elif kind == "t":
+            if i == 0:
+                L += ["s_mov_b32 m0, %[la]", "s_nop 0"]
+            L.append(f"global_load_lds_dwordx4 %[va{i}], %[ap]" + (f" offset:{i * 1024}" if i else ""))
+        else:
+            if i == 0:
+                L += ["s_mov_b32 m0, %[lw]", "s_nop 0"]
+            L.append(f"global_load_lds_dwordx4 %[vw{i}], %[wp]" + (f" offset:{i * 1024}" if i else ""))
+        for _ in range(per):
+            if rd:
+                d, a, off = rd.pop(0)
+                L.append(f"ds_read_b128 {d}, %[{a}]" + (f" offset:{off}" if off else ""))
+    for d, a, off in rd:
+        L.append(f"ds_read_b128 {d}, %[{a}]" + (f" offset:{off}" if off else ""))
+    for nt in range(4):
+        off = (nt & 1) * 256 + (nt >> 1) * 4
+        L.append(f"ds_read_b32 v{p.sfw + nt}, %[sfwl]" + (f" offset:{off}" if off else ""))
+    for mt in range(p.mtw):
+        L.append(f"ds_read_b32 v{p.sfa + mt}, %[sfa{mt}]")
+    L.append("s_waitcnt lgkmcnt(0)")
+    for nt in range(4):
+        L.append(f"v_lshrrev_b32 v{p.sfw + nt}, %[sh], v{p.sfw + nt}")
+    for mt in range(p.mtw):
+        L.append(f"v_lshrrev_b32 v{p.sfa + mt}, %[sh], v{p.sfa + mt}")
+    L.append(f"s_waitcnt vmcnt({p.ntc + 5}) ; explicit")
+    L.append("s_barrier")
+    return L
+
+
+def mx_matrix_phase(p):
+    L = []
+    for j in range(p.mtw * NT):
+        mt, nt = divmod(j, NT)
+        if nt == 0 and mt >= 2:
+            L.append("s_waitcnt lgkmcnt(2)" if mt + 1 < p.mtw else "s_waitcnt lgkmcnt(0)")
+        L.append(f"v_mfma_scale_f32_16x16x128_f8f6f4 %[c{nt}_{mt}], {regs(p.w[nt], 8)}, {regs(p.a[mt % 3], 8)}, %[c{nt}_{mt}], "
+                 f"v{p.sfw + nt}, v{p.sfa + mt} op_sel_hi:[0,0,0]")
+        if nt == 0 and mt + 2 < p.mtw:
+            b = p.a[(mt + 2) % 3]
+            L.append(f"ds_read_b128 {regs(b, 4)}, %[al] offset:{(mt + 2) * 2048}")
+            L.append(f"ds_read_b128 {regs(b + 4, 4)}, %[ah] offset:{(mt + 2) * 2048}")
+    L.append("s_waitcnt vmcnt(4) ; explicit")
+    L.append("s_barrier")
+    return L
+
+
+def emit_mx(name, mtw):
+    p = MxPlan(mtw)
+    lines = ablated(mx_memory_phase(p) + mx_matrix_phase(p))
+    print_body(name, lines)
+    print(f"#define {name}_OUTS " + ", ".join(f'[c{nt}_{mt}] "+v"(acc[{nt}][{mt}])' for mt in range(mtw) for nt in range(NT)))
+    ins = [f'[va{i}] "v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "v"(vw[{i}])' for i in range(4)]
+    ins += ['[vs] "v"(vs)', '[wl] "v"(wl)', '[wh] "v"(wh)', '[al] "v"(al)', '[ah] "v"(ah)', '[sfwl] "v"(sfwl)']
+    ins += [f'[sfa{mt}] "v"(sfal[{mt}])' for mt in range(mtw)]
+    ins += ['[sh] "v"(shift)', '[la] "s"(la)', '[lw] "s"(lw)', '[ls] "s"(ls)', '[ap] "s"(ap)', '[wp] "s"(wp)', '[sp] "s"(sp)']
     print(f"#define {name}_INS " + ", ".join(ins))
     print(f"#define {name}_CLOBBERS " + ", ".join(p.clobbers()))
     print(f"#define {name}_LOWEST_FIXED_VGPR {p.lowest}")
@@ -179,6 +281,7 @@ def main():
     for mtw in (4, 6):
         emit(f"ESMOE_PP{mtw * 2}", mtw, False)
         emit(f"ESMOE_PP{mtw * 2}F", mtw, True)
+        emit_mx(f"ESMOE_PPX{mtw * 2}", mtw)
 
 
 if __name__ == "__main__":

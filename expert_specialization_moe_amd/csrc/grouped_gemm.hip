@@ -41,6 +41,7 @@
 #include <stdint.h>
 
 #include <mutex>
+#include <type_traits>
 
 #include "gemm_args.h"
 #include "mx_phase.h"
@@ -51,6 +52,12 @@
 #endif
 #include "schedule.h"
 #include "swiglu.h"
+
+// 1: the hand-scheduled tall tiles copy weight rows that only one tile reads with the non-temporal hint, 0: never
+// (for measurements)
+#ifndef ESMOE_PP_NT
+#define ESMOE_PP_NT 1
+#endif
 
 namespace esmoe {
 
@@ -519,11 +526,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
       for (int mt = 0; mt < MTW; mt++) {
         uint32_t d;
-        if constexpr (MT == 8 || MT == 16) {
-          // tall tiles start on a 128-row boundary and a wavefront's rows start on a multiple of its
-          // own height (64 or 128): row tile mt adds compile-time offsets
+        if constexpr (MT == 16) {
+          // 256-row tiles start on a 128-row boundary and a wavefront's rows on a multiple of 128: row tile mt adds
+          // compile-time offsets
           d = *(const uint32_t*)(lb + sfa_lane + (mt >> 3) * 512 + (mt & 1) * 256 + ((mt & 7) >> 1) * 4);
-        } else if constexpr (MT == 12) {
+        } else if constexpr (MT == 12 || MT == 8) {
+          // 128- and 192-row tiles may start in the middle of a scale tile (full tiles of 192 rows)
           int ml = (m0 & 127) + mw + mt * 16 + r;
           d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4);
         } else {
@@ -856,36 +864,46 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
 #ifdef ESMOE_TIMELINE
   const uint64_t tl_r0 = __builtin_amdgcn_s_memrealtime(), tl_c0 = __builtin_amdgcn_s_memtime();
 #endif
-  int tslot = 0, wslot = 0, sabuf = 0;   // slots of K block kb: tokens kb % 2, weights kb % 3, scale chunk (kb / 4) % 3
-  for (int kb = 0; kb < KB; kb++) {
-    const int q = kb & 3;
-    const int kbt = kb + 1 < KB ? kb + 1 : KB - 1, kbw = kb + 2 < KB ? kb + 2 : KB - 1;
-    const int chw = (kb >> 2) + 2 < NCH ? (kb >> 2) + 2 : NCH - 1;
-    const int wnext = wslot >= 1 ? wslot - 1 : 2;          // (kb + 2) % 3
-    const int sanext = sabuf >= 1 ? sabuf - 1 : 2;         // (kb / 4 + 2) % 3
-    const uint32_t la = t_dst + (tslot ^ 1) * kTSlot, lw = w_dst + wnext * kWSlot;
-    const uint32_t ls = s_dst + sanext * kSaBuf + q * 256;
-    const uint8_t* ap = a_ptr + (long)kbt * 128;
-    const uint8_t* wp = w_ptr + (long)kbw * 128;
-    const uint8_t* sp = sa_ptr + (long)chw * 16;
-    const uint32_t wl = wfrag + wslot * kWSlot, wh = wl ^ 64;
-    const uint32_t al = afrag + tslot * kTSlot, ah = al ^ 64;
-    const uint32_t sal = sa_rd + sabuf * kSaBuf + q * 4;
-    const uint32_t sbl = sb_rd + kb * 4;
-    const uint32_t vsq = vs[0];
-    if constexpr (MT == 12) {
-      if constexpr (FUSE) asm volatile(ESMOE_PP12F_BODY : ESMOE_PP12F_OUTS : ESMOE_PP12F_INS : ESMOE_PP12F_CLOBBERS);
-      else asm volatile(ESMOE_PP12_BODY : ESMOE_PP12_OUTS : ESMOE_PP12_INS : ESMOE_PP12_CLOBBERS);
-    } else {
-      if constexpr (FUSE) asm volatile(ESMOE_PP8F_BODY : ESMOE_PP8F_OUTS : ESMOE_PP8F_INS : ESMOE_PP8F_CLOBBERS);
-      else asm volatile(ESMOE_PP8_BODY : ESMOE_PP8_OUTS : ESMOE_PP8_INS : ESMOE_PP8_CLOBBERS);
+  // Weight rows that no other tile reads (the expert is one tile high) are copied with the non-temporal hint, so
+  // that their stream leaves L2 to the operands that are shared.  One loop per form: a statement of each kind on
+  // alternative paths of one loop would make the compiler shuffle the accumulators between them.
+  const bool w_once = ESMOE_PP_NT && m0 == 0 && M <= BM;
+  auto k_loop = [&](auto nt_hint) {
+    constexpr bool kNt = decltype(nt_hint)::value;
+    int tslot = 0, wslot = 0, sabuf = 0;   // slots of K block kb: tokens kb % 2, weights kb % 3, scale chunk (kb / 4) % 3
+    for (int kb = 0; kb < KB; kb++) {
+      const int q = kb & 3;
+      const int kbt = kb + 1 < KB ? kb + 1 : KB - 1, kbw = kb + 2 < KB ? kb + 2 : KB - 1;
+      const int chw = (kb >> 2) + 2 < NCH ? (kb >> 2) + 2 : NCH - 1;
+      const int wnext = wslot >= 1 ? wslot - 1 : 2;          // (kb + 2) % 3
+      const int sanext = sabuf >= 1 ? sabuf - 1 : 2;         // (kb / 4 + 2) % 3
+      const uint32_t la = t_dst + (tslot ^ 1) * kTSlot, lw = w_dst + wnext * kWSlot;
+      const uint32_t ls = s_dst + sanext * kSaBuf + q * 256;
+      const uint8_t* ap = a_ptr + (long)kbt * 128;
+      const uint8_t* wp = w_ptr + (long)kbw * 128;
+      const uint8_t* sp = sa_ptr + (long)chw * 16;
+      const uint32_t wl = wfrag + wslot * kWSlot, wh = wl ^ 64;
+      const uint32_t al = afrag + tslot * kTSlot, ah = al ^ 64;
+      const uint32_t sal = sa_rd + sabuf * kSaBuf + q * 4;
+      const uint32_t sbl = sb_rd + kb * 4;
+      const uint32_t vsq = vs[0];
+#define ESMOE_PP_STMT(NAME)                                                                                      \
+  do {                                                                                                           \
+    if constexpr (kNt) asm volatile(NAME##_BODY_NT : NAME##_OUTS : NAME##_INS : NAME##_CLOBBERS);                 \
+    else asm volatile(NAME##_BODY : NAME##_OUTS : NAME##_INS : NAME##_CLOBBERS);                                  \
+  } while (0)
+      if constexpr (MT == 12 && FUSE) ESMOE_PP_STMT(ESMOE_PP12F);
+      else if constexpr (MT == 12) ESMOE_PP_STMT(ESMOE_PP12);
+      else if constexpr (FUSE) ESMOE_PP_STMT(ESMOE_PP8F);
+      else ESMOE_PP_STMT(ESMOE_PP8);
+      // the piece offsets rotate with q; slots advance
+      { const uint32_t t = vs[0]; vs[0] = vs[1]; vs[1] = vs[2]; vs[2] = vs[3]; vs[3] = t; }
+      tslot ^= 1;
+      wslot = wslot == 2 ? 0 : wslot + 1;
+      if (q == 3) sabuf = sabuf == 2 ? 0 : sabuf + 1;
     }
-    // the piece offsets rotate with q; slots advance
-    { const uint32_t t = vs[0]; vs[0] = vs[1]; vs[1] = vs[2]; vs[2] = vs[3]; vs[3] = t; }
-    tslot ^= 1;
-    wslot = wslot == 2 ? 0 : wslot + 1;
-    if (q == 3) sabuf = sabuf == 2 ? 0 : sabuf + 1;
-  }
+  };
+  if (w_once) k_loop(std::true_type{}); else k_loop(std::false_type{});
 #ifdef ESMOE_TIMELINE
   if (timeline && tid == 0) {   // debug build: K loop start and end (100 MHz ticks), its length in shader clocks
     timeline[4] = (uint32_t)tl_r0;
@@ -898,6 +916,160 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
   if (grp == 0) block_barrier();
   block_barrier();
   tile_epilogue<BM, MTW, NTW, 4, FUSE>(g, acc, M, m0, n0, row_base, mw, nw, wj, lane, wave_active, lds);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Tall mxfp8 tiles (MT = 8 or 12): the same two-group schedule and split ring as gemm_tile_pp with the scaled MFMA.
+//
+//   LDS   3 weight slots of 32 KB + 1 KB (the K block's two 512-byte scale tiles of the tile's 256 weight rows)
+//         4 token regions (group g, 2 slots) of GR rows x 128 B + 1 KB (the two scale tiles that hold the group's rows)
+//         1 KB spare, the target of the scale copies of the wavefronts that have no scale tile to fetch
+// A tile may start in the middle of a 128-row scale tile (full tiles are 192 rows): a lane finds the scale dword of
+// its row from the row's position inside the two tiles that were fetched for its group.
+template <int MT>
+__device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds,
+                                                uint32_t* timeline = nullptr) {
+  static_assert(MT == 8 || MT == 12, "hand-scheduled K block: 128- and 192-row tiles");
+  constexpr int MTW = MT / 2, NTW = 4, BM = MT * 16, GR = MTW * 16;
+  constexpr int kTCopies = MTW / 2;
+  constexpr int kWSlot = kBN * 128 + 1024, kTSlot = GR * 128 + 1024;
+  constexpr int kTBase = 3 * kWSlot, kSpare = kTBase + 4 * kTSlot;
+  static_assert(kSpare + 1024 <= kLdsBytes, "LDS map of the split ring");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2, wj = wave & 3;
+  const int r = lane & 15, gq = lane >> 4;
+  const int K = g.k, N = g.n, KB = K >> 7, kc = K >> 5;
+  const long row_base = g.expert_offsets[e];
+  const int nw = wj * 64, mw = grp * GR;
+  const bool wave_active = n0 + nw < N;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
+
+  // ---- copy plan --------------------------------------------------------------------------------------------
+  constexpr int kBias = 3072;
+  const int crow = lane >> 3, cslot = lane & 7;
+  const int a_last = M - 1 - m0;
+  uint32_t va[kTCopies], vw[4];
+#pragma unroll
+  for (int i = 0; i < kTCopies; i++) {
+    const int lrow = (wj * kTCopies + i) * 8 + crow;
+    const int trow = mw + lrow;
+    const int grow = trow > a_last ? a_last : trow;
+    va[i] = (uint32_t)grow * (uint32_t)K + (swz(lrow, cslot) << 4) + kBias - i * 1024;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int blk = wave * 4 + i;
+    const int row = (n0 + blk * 8 < N ? blk : i) * 8;
+    vw[i] = (uint32_t)(row + crow) * (uint32_t)K + (swz(blk * 8 + crow, cslot) << 4) + kBias - i * 1024;
+  }
+  const uint8_t* a_ptr = (const uint8_t*)g.a + (row_base + m0) * K - kBias;
+  const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + n0) * K - kBias;
+  const uint32_t t_dst = lds0 + kTBase + grp * 2 * kTSlot + wj * kTCopies * 1024;   // + slot * kTSlot
+  const uint32_t w_dst = lds0 + wave * 4096;                                        // + slot * kWSlot
+  // scale copies, one per wavefront and K block: wavefront 0 the weight scale tiles (with the weight stage),
+  // wavefronts 1 and 5 their group's token scale tiles (with the token stage), the others one line into the spare
+  const int s_role = wave == 0 ? 0 : (wj == 1 ? 1 : 2);
+  const uint8_t* s_ptr;
+  uint32_t vs, s_dst;
+  const int tblk0 = (m0 + mw) >> 7;          // first 128-row scale tile of the group's rows inside the expert
+  if (s_role == 0) {
+    int blk = (n0 >> 7) + (lane >> 5);
+    if (blk * 128 >= N) blk = n0 >> 7;
+    s_ptr = g.sfb + (long)e * N * kc;
+    vs = (uint32_t)blk * (uint32_t)KB * 512 + (lane & 31) * 16;
+    s_dst = lds0 + kBN * 128;                // + slot * kWSlot
+  } else if (s_role == 1) {
+    int blk = tblk0 + (lane >> 5);
+    if (blk * 128 >= M) blk = tblk0 * 128 < M ? tblk0 : m0 >> 7;
+    s_ptr = g.sfa + (long)g.blockscale_offsets[e] * kc;
+    vs = (uint32_t)blk * (uint32_t)KB * 512 + (lane & 31) * 16;
+    s_dst = lds0 + kTBase + grp * 2 * kTSlot + GR * 128;   // + slot * kTSlot
+  } else {
+    s_ptr = g.sfb + (long)e * N * kc;
+    vs = 0;
+    s_dst = lds0 + kSpare;
+  }
+  // (wave-uniform by construction; said again so that they live in scalar registers)
+  s_dst = __builtin_amdgcn_readfirstlane(s_dst);
+  s_ptr = (const uint8_t*)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)((uint64_t)s_ptr >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint64_t)s_ptr));
+  auto issue_t = [&](int kb, int slot) { dma16xn<false>(t_dst + slot * kTSlot, a_ptr + (long)kb * 128, va); };
+  auto issue_w = [&](int kb, int slot) { dma16xn<false>(w_dst + slot * kWSlot, w_ptr + (long)kb * 128, vw); };
+  auto issue_s = [&](int kb, int slot) {
+    dma16(s_ptr + (long)kb * 512, vs, s_dst + (s_role == 0 ? slot * kWSlot : s_role == 1 ? slot * kTSlot : 0));
+  };
+
+  // ---- fragment and scale read plan -------------------------------------------------------------------------
+  const uint32_t wfrag = lds0 + (nw + r) * 128 + swz(r, gq) * 16;                       // + slot * kWSlot
+  const uint32_t afrag = lds0 + kTBase + grp * 2 * kTSlot + r * 128 + swz(r, gq) * 16;  // + slot * kTSlot
+  // weight scale dword of row nw + nt*16 + r: n-tile nt at + (nt & 1)*256 + (nt >> 1)*4
+  const uint32_t sfw_rd = lds0 + kBN * 128 + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16;
+  uint32_t sfa_rd[MTW];
+#pragma unroll
+  for (int mt = 0; mt < MTW; mt++) {
+    const int ml = ((m0 + mw) & 127) + mt * 16 + r;   // row inside the group's two scale tiles
+    sfa_rd[mt] = lds0 + kTBase + grp * 2 * kTSlot + GR * 128 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4;
+  }
+  const uint32_t shift = gq * 8;
+
+  v4f acc[NTW][MTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) acc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // ---- prologue: scale tiles and stages of K blocks 0 (tokens, weights) and 1 (weights) ------------------------
+  const int kb1 = 1 < KB ? 1 : KB - 1;
+  issue_s(0, 0);
+  if (s_role == 0) issue_s(kb1, 1); else issue_s(0, 0);
+  issue_t(0, 0);
+  issue_w(0, 0);
+  issue_w(kb1, 1);
+  wait_vmcnt<4>();
+  block_barrier();
+  if (grp == 1) block_barrier();
+
+#ifdef ESMOE_TIMELINE
+  const uint64_t tl_r0 = __builtin_amdgcn_s_memrealtime(), tl_c0 = __builtin_amdgcn_s_memtime();
+#endif
+  const bool w_once = ESMOE_PP_NT && m0 == 0 && M <= BM;   // nobody else reads these weight rows: non-temporal copies (see gemm_tile_pp)
+  auto k_loop = [&](auto nt_hint) {
+    constexpr bool kNt = decltype(nt_hint)::value;
+    int tslot = 0, wslot = 0;
+    for (int kb = 0; kb < KB; kb++) {
+      const int kbt = kb + 1 < KB ? kb + 1 : KB - 1, kbw = kb + 2 < KB ? kb + 2 : KB - 1;
+      const int wnext = wslot >= 1 ? wslot - 1 : 2;          // (kb + 2) % 3
+      const uint32_t la = t_dst + (tslot ^ 1) * kTSlot, lw = w_dst + wnext * kWSlot;
+      const uint32_t ls = s_dst + (s_role == 0 ? wnext * kWSlot : s_role == 1 ? (tslot ^ 1) * kTSlot : 0);
+      const uint8_t* ap = a_ptr + (long)kbt * 128;
+      const uint8_t* wp = w_ptr + (long)kbw * 128;
+      const uint8_t* sp = s_ptr + (long)(s_role == 0 ? kbw : kbt) * 512;
+      const uint32_t wl = wfrag + wslot * kWSlot, wh = wl ^ 64;
+      const uint32_t al = afrag + tslot * kTSlot, ah = al ^ 64;
+      const uint32_t sfwl = sfw_rd + wslot * kWSlot;
+      uint32_t sfal[MTW];
+#pragma unroll
+      for (int mt = 0; mt < MTW; mt++) sfal[mt] = sfa_rd[mt] + tslot * kTSlot;
+      if constexpr (MT == 12) ESMOE_PP_STMT(ESMOE_PPX12);
+      else ESMOE_PP_STMT(ESMOE_PPX8);
+      tslot ^= 1;
+      wslot = wslot == 2 ? 0 : wslot + 1;
+    }
+  };
+  if (w_once) k_loop(std::true_type{}); else k_loop(std::false_type{});
+#ifdef ESMOE_TIMELINE
+  if (timeline && tid == 0) {
+    timeline[4] = (uint32_t)tl_r0;
+    timeline[5] = (uint32_t)__builtin_amdgcn_s_memrealtime();
+    timeline[6] = (uint32_t)(__builtin_amdgcn_s_memtime() - tl_c0);
+  }
+#endif
+  wait_vmcnt<0>();
+  if (grp == 0) block_barrier();
+  block_barrier();
+  tile_epilogue<BM, MTW, NTW, 4, false>(g, acc, M, m0, n0, row_base, mw, nw, wj, lane, wave_active, lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -968,6 +1140,10 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 // Heights whose fp8-blockwise tiles run the hand-scheduled K block of gemm_tile_pp (bit 0: 128 rows, bit 1: 192 rows).
 #ifndef ESMOE_PP_HEIGHTS
 #define ESMOE_PP_HEIGHTS 3
+#endif
+// The same for mxfp8 tiles (gemm_tile_pp_mx).
+#ifndef ESMOE_PPX_HEIGHTS
+#define ESMOE_PPX_HEIGHTS 3
 #endif
 // Tile heights (MT * 16 rows) compiled into the persistent kernel.
 #ifndef ESMOE_VARIANTS
@@ -1065,6 +1241,15 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
 #endif
     // tall fp8-blockwise tiles take the hand-scheduled K block when the scale chunks fit K (a multiple of 512)
     bool hand_scheduled = false;
+    if constexpr (MX) {
+      if ((ESMOE_PPX_HEIGHTS & 2) && t.mt == 12) {
+        gemm_tile_pp_mx<12>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        hand_scheduled = true;
+      } else if ((ESMOE_PPX_HEIGHTS & 1) && t.mt == 8) {
+        gemm_tile_pp_mx<8>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        hand_scheduled = true;
+      }
+    }
     if constexpr (!MX) {
       if ((g.k & 511) == 0) {
         if ((ESMOE_PP_HEIGHTS & 2) && t.mt == 12) {

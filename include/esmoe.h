@@ -231,8 +231,8 @@ int esmoe_permute_rows(const void* in, const int32_t* dst_row, long num_pairs, i
  * expert's tile grid (the kernel skips it), or 2 if that XCD's queue is exhausted.
  * The other experts are "light": one short tile per 256 columns from a launch-wide counter;
  * esmoe_host_decode_light maps item `item` (< word 1 of the workspace) to out5.
- * mx: 0 describes the FP8-blockwise launch (full tiles of 192 rows), 1 the MXFP8 launch (256 rows).  The mirrors
- * describe the default policy; the ESMOE_* environment variables, which a launch reads once per process, do not
+ * mx: 0 describes the FP8-blockwise launch, 1 the MXFP8 launch (both cut experts into full tiles of 192 rows today).
+ * The mirrors describe the default policy; the ESMOE_* environment variables, which a launch reads once per process, do not
  * reach them.
  */
 int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int mx,

@@ -56,22 +56,21 @@ def test_tiles_cover_every_output_element_exactly_once(esmoe, force_bm, n, mx):
             assert bm == force_bm
         cover[e][m0:m0 + bm, n0:n0 + bn] += 1
         if not force_bm:
-            # full tiles: 192 rows for fp8-blockwise, 256 for mxfp8, then one remainder tile
-            assert bm <= (256 if mx else 192)
-            assert m0 % (256 if mx else 192) == 0
-        if mx and bm in (128, 256):
-            # the mxfp8 kernel reads the token scales of these heights assuming a start on a scale-tile boundary
+            # full tiles of 192 rows for both kernels, then one remainder tile
+            assert bm <= 192 and m0 % 192 == 0
+        if mx and bm == 256:
+            # the mxfp8 kernel reads the token scales of 256-row tiles assuming a start on a scale-tile boundary
             assert m0 % 128 == 0
     for c in cover:
         assert (c == 1).all()
 
 
-def test_mx_policy_uses_256_row_full_tiles(esmoe):
+def test_both_kernels_use_192_row_full_tiles(esmoe):
     from expert_specialization_moe_amd import _native
 
     heights = lambda mx: sorted({t[1] for t in _schedule(_native, [700], 256, 0, mx=mx)})
     assert heights(0) == [128, 192]      # 3 x 192 + 124 -> 128
-    assert heights(1) == [192, 256]      # 2 x 256 + 188 -> 192
+    assert heights(1) == [128, 192]
 
 
 def test_auto_shapes_waste_less_than_any_single_shape(esmoe):
