@@ -94,8 +94,8 @@ const Knobs& knobs() {
     const char* big = getenv("ESMOE_BIG_MT");
     if (big && *big) {
       const int v = atoi(big);
-      if (v == 8 || v == 12 || v == 16) r.big_mt_fp8 = r.big_mt_mx = v;
-      else snprintf(r.error, sizeof(r.error), "ESMOE_BIG_MT=%s: full tiles are 8, 12 or 16 x 16 rows", big);
+      if (v == 8 || v == 12) r.big_mt_fp8 = r.big_mt_mx = v;
+      else snprintf(r.error, sizeof(r.error), "ESMOE_BIG_MT=%s: full tiles are 8 or 12 x 16 rows", big);
     }
     r.order = env_int("ESMOE_ORDER", 0);
     if (r.order < 0 || r.order > 2) snprintf(r.error, sizeof(r.error), "ESMOE_ORDER must be 0, 1 or 2");
@@ -113,8 +113,8 @@ esmoe::SchedPolicy default_policy(int force_bm, int mx) {
   esmoe::SchedPolicy p;
   p.force_mt = force_bm / 16;
   // Full tiles are 192 rows for both kernels: the tallest tile whose ring (three weight stages, two token stages per
-  // wavefront group) fits the 160 KB of LDS, which is what the hand-scheduled K block of the tall tiles needs; 256-row
-  // tiles do more MFMA work per byte copied but run with a two-stage ring and measured slower.
+  // wavefront group) fits the 160 KB of LDS, which is what the hand-scheduled K block of the tall tiles needs.  (A
+  // 256-row tile does more MFMA work per byte copied but only fits with two stages per operand and measured slower.)
   (void)mx;
   p.big_mt = 12;
   p.order = 0;
@@ -143,9 +143,8 @@ int check_common(const void* out, const void* a, const void* b, const int32_t* p
   if (total_rows < 0) return fail(ESMOE_ERR_INVALID_ARGUMENT, "total_rows must be >= 0");
   if (out_dtype != ESMOE_OUT_BF16 && out_dtype != ESMOE_OUT_FP16)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "out_dtype must be ESMOE_OUT_BF16 or ESMOE_OUT_FP16");
-  if (force_bm != 0 && force_bm != 16 && force_bm != 32 && force_bm != 64 && force_bm != 128 && force_bm != 192 &&
-      force_bm != 256)
-    return fail(ESMOE_ERR_INVALID_ARGUMENT, "force_bm must be 0, 16, 32, 64, 128, 192 or 256, got %d", force_bm);
+  if (force_bm != 0 && force_bm != 16 && force_bm != 32 && force_bm != 64 && force_bm != 128 && force_bm != 192)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "force_bm must be 0, 16, 32, 64, 128 or 192, got %d", force_bm);
   if (!workspace || workspace_bytes < esmoe_gemm_workspace_bytes(num_experts))
     return fail(ESMOE_ERR_WORKSPACE_TOO_SMALL, "workspace of %zu bytes is smaller than the %zu required",
                 workspace_bytes, esmoe_gemm_workspace_bytes(num_experts));

@@ -774,7 +774,10 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave >> 2, wj = wave & 3;
   const int r = lane & 15, gq = lane >> 4;
-  const int K = g.k, N = g.n, KB = K >> 7, NCH = KB >> 2;
+  // Scale chunk c holds sa of K blocks first_kb(c) .. + 3, first_kb(c) = min(4c, KB - 4) clamped at 0: the last chunk of
+  // a K that is no multiple of 512 overlaps the one before instead of reaching past the row.
+  const int K = g.k, N = g.n, KB = K >> 7, NCH = (KB + 3) >> 2;
+  auto chunk_first_kb = [&](int c) { const int f = 4 * c < KB - 4 ? 4 * c : KB - 4; return f > 0 ? f : 0; };
   const long row_base = g.expert_offsets[e];
   const int nw = wj * 64, mw = grp * GR;
   const bool wave_active = n0 + nw < N;
@@ -811,7 +814,7 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
   for (int q = 0; q < 4; q++) {
     const int trow = mw + (wj & 1) * 64 + q * 16 + (lane >> 2);
     const int grow = trow > a_last ? a_last : trow;
-    vs[q] = (uint32_t)grow * (uint32_t)KB * 4 + (lane & 3) * 4;
+    vs[q] = (uint32_t)grow * (uint32_t)KB * 4 + ((lane & 3) < KB ? (lane & 3) : KB - 1) * 4;
   }
   const uint8_t* a_ptr = (const uint8_t*)g.a + (row_base + m0) * K - kBias;
   const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + (FUSE ? 0 : n0)) * K - kBias;
@@ -848,11 +851,12 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
     }
   }
   {
-    // chunk (wj >> 1), rows (wj & 1)*64 + lane of the group: 16 bytes per row
+    // scale chunks 0 and 1 in the pieces the loop uses: wavefront wj the four 16-row pieces of rows (wj & 1)*64 .. +64
+    // of chunk wj >> 1
     const int ch = (wj >> 1) < NCH ? (wj >> 1) : NCH - 1;
-    const int trow = mw + (wj & 1) * 64 + lane;
-    const int grow = trow > a_last ? a_last : trow;
-    dma16(sa_ptr + (long)ch * 16, (uint32_t)grow * (uint32_t)KB * 4, lds0 + kSaBase + (grp * 3 + (wj >> 1)) * kSaBuf + (wj & 1) * 1024);
+    const uint8_t* src = sa_ptr + (long)chunk_first_kb(ch) * 4;
+#pragma unroll
+    for (int q = 0; q < 4; q++) dma4(src, vs[q], s_dst + (wj >> 1) * kSaBuf + q * 256);
   }
   issue_t(0, 0);
   issue_w(0, 0);
@@ -881,10 +885,10 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
       const uint32_t ls = s_dst + sanext * kSaBuf + q * 256;
       const uint8_t* ap = a_ptr + (long)kbt * 128;
       const uint8_t* wp = w_ptr + (long)kbw * 128;
-      const uint8_t* sp = sa_ptr + (long)chw * 16;
+      const uint8_t* sp = sa_ptr + (long)chunk_first_kb(chw) * 4;
       const uint32_t wl = wfrag + wslot * kWSlot, wh = wl ^ 64;
       const uint32_t al = afrag + tslot * kTSlot, ah = al ^ 64;
-      const uint32_t sal = sa_rd + sabuf * kSaBuf + q * 4;
+      const uint32_t sal = sa_rd + sabuf * kSaBuf + (kb - chunk_first_kb(kb >> 2)) * 4;
       const uint32_t sbl = sb_rd + kb * 4;
       const uint32_t vsq = vs[0];
 #define ESMOE_PP_STMT(NAME)                                                                                      \
@@ -1147,7 +1151,7 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
 #endif
 // Tile heights (MT * 16 rows) compiled into the persistent kernel.
 #ifndef ESMOE_VARIANTS
-#define ESMOE_VARIANTS ESMOE_CASE(1) ESMOE_CASE(2) ESMOE_CASE(4) ESMOE_CASE(8) ESMOE_CASE(12) ESMOE_CASE(16)
+#define ESMOE_VARIANTS ESMOE_CASE(1) ESMOE_CASE(2) ESMOE_CASE(4)
 #endif
 
 template <bool MX, bool FUSE>
@@ -1169,8 +1173,9 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   const bool light_first = (int)(blockIdx.x / kXcds) * 32 / per_xcd >= 32 - ws[kWsLightShare];
   int phase = 0, q = 0;
   // Queues known to be exhausted (bits 0-7: the XCDs' heavy queues, bit 8: the light items).  When a draw comes back
-  // past the end of its queue, one look at all nine counters marks every queue that has run dry, so that a workgroup
-  // leaving its own queue does not spend an atomic round trip (about a microsecond under load) on each empty one.
+  // past the end of its queue and the launch has heavy blocks on every XCD, one look at all nine counters marks every
+  // queue that has run dry, so that a workgroup leaving its own queue does not spend an atomic round trip (about a
+  // microsecond under load) on each empty one.
   int dead = ltotal == 0 ? 256 : 0;
 #pragma unroll
   for (int x = 0; x < kXcds; x++)
@@ -1203,6 +1208,8 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     if (v >= (light ? ltotal : hblocks)) {   // this queue is exhausted: see which others are
       dead |= 1 << (light ? 8 : xq);
       __syncthreads();                        // s_item and s_counters are rewritten next
+      // (worth its round trip only when every XCD has a queue to try: the look itself reads the hot counter line)
+      if (hblocks <= kXcds) continue;
       if (threadIdx.x < kXcds + 1)
         s_counters[threadIdx.x] = __hip_atomic_load(threadIdx.x < kXcds ? &ws[kWsXcdCounter + threadIdx.x] : &ws[kWsLightCounter],
                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1251,14 +1258,12 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
       }
     }
     if constexpr (!MX) {
-      if ((g.k & 511) == 0) {
-        if ((ESMOE_PP_HEIGHTS & 2) && t.mt == 12) {
-          gemm_tile_pp<12, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
-          hand_scheduled = true;
-        } else if ((ESMOE_PP_HEIGHTS & 1) && t.mt == 8) {
-          gemm_tile_pp<8, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
-          hand_scheduled = true;
-        }
+      if ((ESMOE_PP_HEIGHTS & 2) && t.mt == 12) {
+        gemm_tile_pp<12, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        hand_scheduled = true;
+      } else if ((ESMOE_PP_HEIGHTS & 1) && t.mt == 8) {
+        gemm_tile_pp<8, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        hand_scheduled = true;
       }
     }
     if (!hand_scheduled) {

@@ -54,7 +54,7 @@ size_t esmoe_gemm_workspace_bytes(int num_experts);
  *   sa   [total_rows, K/128] fp32;  sb [E, N/128, K/128] fp32
  * N % 128 == 0, K % 128 == 0, 1 <= E <= ESMOE_MAX_EXPERTS.
  * force_bm: 0 lets the device-side schedule pick an M-tile shape per expert;
- *           16/32/64/128/192/256 forces that single shape for every tile (benchmarking).
+ *           16/32/64/128/192 forces that single shape for every tile (benchmarking).
  * Rows of `out` that belong to no expert (M_e == 0) are not written.
  */
 int esmoe_fp8_blockwise_grouped_mm(void* out, int out_dtype, const void* a, const void* b, const float* sa,

@@ -27,7 +27,7 @@ def _fused(native, ops, inter, mid_dtype, force_bm=0, q=None, sc=None):
     return q, sc
 
 
-@pytest.mark.parametrize("force_bm", [0, 16, 32, 64, 128, 192, 256])
+@pytest.mark.parametrize("force_bm", [0, 16, 32, 64, 128, 192])
 @pytest.mark.parametrize("mid_dtype", [torch.bfloat16, torch.float16])
 def test_fused_equals_projection_then_swiglu_quant(esmoe, force_bm, mid_dtype):
     """Bit-exact against this library's own separate route: grouped GEMM into `mid_dtype`, then the fused
