@@ -14,8 +14,9 @@ struct GemmArgs {
   const uint8_t* sfa;   // mxfp8: swizzled E8M0, expert base blockscale_offsets[e] * K/32
   const uint8_t* sfb;   // mxfp8: swizzled E8M0, expert base e * N * K/32
   void* out;            // [total_rows, N]
-  void* q_out;          // fused SwiGLU + quantisation (fp8-blockwise): e4m3 [total_rows, N/2]; null = plain projection
-  float* scales_out;    //   and its fp32 scales [total_rows, N/256]
+  void* q_out;          // fused SwiGLU + quantisation: e4m3 [total_rows, N/2]; null = plain projection
+  float* scales_out;    //   fp8-blockwise: its fp32 scales [total_rows, N/256]
+  uint8_t* sf_out;      //   mxfp8: its swizzled E8M0 scales, expert base blockscale_offsets[e] * N/64
   const int32_t* problem_sizes;
   const int32_t* expert_offsets;
   const int32_t* blockscale_offsets;

@@ -187,8 +187,9 @@ def emit(name, mtw, fuse):
 # kb + 2, wavefronts 1 and 5: their group's token scales of kb + 1, the others re-read one line into a spare area).
 # A lane reads the scale dword of its row and shifts its K sub-block's byte (lane / 16) down to byte 0.
 class MxPlan:
-    def __init__(self, mtw):
+    def __init__(self, mtw, fuse=False):
         self.mtw = mtw
+        self.fuse = fuse                    # gate_up weights: n-tiles 0, 1 are gate rows, 2, 3 the matching up rows
         self.w = [224 + 8 * n for n in range(4)]
         self.a = [200, 208, 216]
         self.sfw = 196                      # 4 weight-row scale registers
@@ -228,7 +229,8 @@ def mx_memory_phase(p):
     for d, a, off in rd:
         L.append(f"ds_read_b128 {d}, %[{a}]" + (f" offset:{off}" if off else ""))
     for nt in range(4):
-        off = (nt & 1) * 256 + (nt >> 1) * 4
+        # plain: n-tiles 2, 3 are the next 32-row quarter of the same scale tile; gate_up: the second tile (up rows)
+        off = (nt & 1) * 256 + (nt >> 1) * (512 if p.fuse else 4)
         L.append(f"ds_read_b32 v{p.sfw + nt}, %[sfwl]" + (f" offset:{off}" if off else ""))
     for mt in range(p.mtw):
         L.append(f"ds_read_b32 v{p.sfa + mt}, %[sfa{mt}]")
@@ -259,8 +261,8 @@ def mx_matrix_phase(p):
     return L
 
 
-def emit_mx(name, mtw):
-    p = MxPlan(mtw)
+def emit_mx(name, mtw, fuse=False):
+    p = MxPlan(mtw, fuse)
     lines = ablated(mx_memory_phase(p) + mx_matrix_phase(p))
     print_body(name, lines)
     print(f"#define {name}_OUTS " + ", ".join(f'[c{nt}_{mt}] "+v"(acc[{nt}][{mt}])' for mt in range(mtw) for nt in range(NT)))
@@ -282,6 +284,7 @@ def main():
         emit(f"ESMOE_PP{mtw * 2}", mtw, False)
         emit(f"ESMOE_PP{mtw * 2}F", mtw, True)
         emit_mx(f"ESMOE_PPX{mtw * 2}", mtw)
+        emit_mx(f"ESMOE_PPX{mtw * 2}F", mtw, True)
 
 
 if __name__ == "__main__":

@@ -1,42 +1,36 @@
 // Persistent grouped GEMM for gfx950 (MI355X): FP8-blockwise and MXFP8 variants.
 //
-// One launch serves every expert.  A one-workgroup schedule kernel turns
-// problem_sizes into a list of workgroup tiles (schedule.h); persistent workgroups
-// of 8 wavefronts then pull tiles from an atomic counter.  A tile is (MT*16) token
-// rows x 256 weight rows.
+// One launch serves every expert.  A one-workgroup schedule kernel turns problem_sizes into a list of workgroup
+// tiles (schedule.h); persistent workgroups of 8 wavefronts then pull tiles from atomic counters.  A tile is
+// (MT*16) token rows x 256 weight rows, MT in {1, 2, 4} (short tiles, gemm_tile) or {8, 12} (tall tiles,
+// gemm_tile_pp / gemm_tile_pp_mx).
 //
-// Data movement.  Per 128-wide K block the workgroup copies the token rows, the
-// weight rows and the block's scales of its tile from global memory straight into
-// an LDS ring with global_load_lds (no staging registers, no LDS store
-// instructions).  One wavefront instruction moves 8 rows x 128 bytes: 8 consecutive
-// lanes read one row's 128 contiguous bytes, and LDS receives the 64 lanes' 16-byte
-// chunks back to back.  The ring holds 2..4 K blocks depending on the tile height
-// (148 KB of the 160 KB LDS), so up to 3 K blocks of loads are in flight per
-// workgroup; with a loaded-memory latency near 2 us that ring, not the matrix pipe,
-// bounds the tall tiles.  LDS rows are 128 bytes apart; chunk c of row r is stored in
-// 16-byte slot c ^ ((r >> 1) & 7), which makes the MFMA fragment reads (16 rows x 16
-// bytes per quarter-wave) bank-conflict free.  Loading fragments straight from global
-// memory is ~4x slower per CU: a fragment puts consecutive lanes on different rows,
-// i.e. 64 separate 16-byte requests per instruction.
+// Data movement.  Per 128-wide K block the workgroup copies the token rows, the weight rows and the block's scales
+// of its tile from global memory straight into LDS with global_load_lds (no staging registers, no LDS store
+// instructions).  One wavefront instruction moves 8 rows x 128 bytes: 8 consecutive lanes read one row's 128
+// contiguous bytes, and LDS receives the 64 lanes' 16-byte chunks back to back.  LDS rows are 128 bytes apart; chunk
+// c of row r is stored in 16-byte slot c ^ ((r >> 1) & 7), which makes the MFMA fragment reads (16 rows x 16 bytes
+// per quarter-wave) bank-conflict free.  Loading fragments straight from global memory is ~4x slower per CU: a
+// fragment puts consecutive lanes on different rows, i.e. 64 separate 16-byte requests per instruction.
 //
-// K loop.  Tiles whose fragments fit in registers (up to 192 rows) split each K block
-// in a read phase (LDS -> registers) and an MFMA phase, and run the two groups of four
-// wavefronts half an iteration apart: one group's fragment reads overlap the other
-// group's MFMAs.  Copies are issued in groups that share one write of m0 and use the
-// instruction's immediate offset.
+// Short tiles (up to 64 rows, bound by streaming their weight rows from HBM): a ring of up to 4 whole K-block
+// stages (148 KB), every wavefront owns all token rows and 32 weight rows, compiler-scheduled K loop.
+// Tall tiles (128 and 192 rows, bound by the matrix pipe and its feed): the K block is ONE hand-scheduled statement
+// (pp_phase.h, written by gen_pp_phase.py); two groups of four wavefronts, one of each per SIMD, run half a K block
+// apart, so that one group's copies and fragment reads overlap the other group's MFMAs; the ring is split by
+// operand (three weight stages shared by both groups, two token stages per group).
 //
 // MFMA mapping (v_mfma[_scale]_f32_16x16x128_f8f6f4, both operands e4m3):
-//   * the weight rows ride on the instruction's "A" side and the token rows on its
-//     "B" side, so a lane ends up with 4 consecutive output columns of one token
-//     row (one packed 8-byte store);
-//   * lane l feeds row (l % 16); its 8 operand registers hold K bytes
-//     [16*(l/16), +16) and [64 + 16*(l/16), +16) of the 128-wide K block;
-//   * for the scaled form lane l supplies the E8M0 scale of row (l % 16),
-//     K sub-block (l / 16) in byte 0 of the scale register.
+//   * the weight rows ride on the instruction's "A" side and the token rows on its "B" side, so a lane ends up with
+//     4 consecutive output columns of one token row (one packed 8-byte store);
+//   * lane l feeds row (l % 16); its 8 operand registers hold K bytes [16*(l/16), +16) and [64 + 16*(l/16), +16)
+//     of the 128-wide K block;
+//   * for the scaled form lane l supplies the E8M0 scale of row (l % 16), K sub-block (l / 16) in byte 0 of the
+//     scale register.
 //
-// FP8-blockwise arithmetic follows the reference's blockwise mainloop order
-// (es_fp8_blockwise_traits.cuh:35,60): each 128-wide K block is multiplied into a
-// zeroed temporary and promoted into the fp32 accumulator times sa[row]*sb[nblk].
+// FP8-blockwise arithmetic follows the reference's blockwise mainloop order (es_fp8_blockwise_traits.cuh:35,60):
+// each 128-wide K block is multiplied into a zeroed temporary and promoted into the fp32 accumulator times
+// sa[row]*sb[nblk].
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -44,7 +38,7 @@
 #include <type_traits>
 
 #include "gemm_args.h"
-#include "mx_phase.h"
+#include "mx_scale.h"
 #ifdef ESMOE_PP_HEADER
 #include ESMOE_PP_HEADER
 #else
@@ -146,13 +140,12 @@ __device__ __forceinline__ void block_barrier() {
   asm volatile("" ::: "memory");
 }
 
-// Shape of a tile with MT*16 token rows and the layout of one ring stage (token rows, weight rows,
-// scales).  Tall tiles (MT >= 8) split the wavefronts 2 (token rows) x 4 (weight rows); short tiles
-// give each of the 8 wavefronts all token rows and 32 weight rows.
+// Shape of a short tile (MT*16 <= 64 token rows) and the layout of one ring stage (token rows, weight rows, scales):
+// each of the 8 wavefronts has all token rows and 32 weight rows.  (Tall tiles: gemm_tile_pp, gemm_tile_pp_mx.)
 template <int MT, bool MX>
 struct TileGeom {
   static constexpr int BM = MT * 16;
-  static constexpr int kWavesM = MT >= 8 ? 2 : 1;
+  static constexpr int kWavesM = 1;
   static constexpr int kWavesN = kWaves / kWavesM;
   static constexpr int MTW = MT / kWavesM;          // row tiles per wavefront
   static constexpr int NTW = kBN / 16 / kWavesN;    // weight-row tiles per wavefront
@@ -263,13 +256,96 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, Acc& acc, int M
   }
 }
 
-// FUSE (fp8-blockwise only): the weights are a gate_up projection [E, 2I, K] (gate rows first) and the tile's 256
-// weight rows are 128 gate rows and the matching 128 up rows, interleaved so that every wavefront holds gate and up
-// of the same columns; the epilogue forms silu(gate) * up and quantises the 128-wide block (one scale per row),
-// writing e4m3 bytes and fp32 scales instead of the bf16 projection.
+// Fused epilogue of an mxfp8 gate_up projection: SwiGLU and the 1x32 E8M0 quantisation of the result, the operand
+// format of the down projection: e4m3 bytes [total_rows, I] and scale bytes in the swizzled 512-byte tiles (128 rows x 4
+// scale columns) of an operand with K = I, expert base blockscale_offsets[e] * I/32.  The arithmetic and its order are
+// those of the unfused sequence (projection rounded to the output type, silu(gate) * up in fp32 rounded to the output
+// type, block maximum, power-of-two scale, e4m3), so the bytes are the same.  A wavefront holds NTW/2 * 16 h columns of
+// its rows: one whole 1x32 block on tall tiles, half of one on short tiles, where two neighbouring wavefronts exchange
+// their maxima through LDS.  Scale bytes of the rows between the expert's last row and the end of its last 128-row
+// scale tile are written as 0, as the stand-alone quantisation does.
+template <int BM, int MTW, int NTW, int kWavesN, typename Acc>
+__device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, int e, int M, int m0, int n0,
+                                                  long row_base, int mw, int wn, int lane, uint8_t* lds) {
+  constexpr int kHalf = NTW / 2, kRW = NTW * 16;
+  constexpr bool kPair = kHalf == 1;
+  static_assert(kHalf == 1 || kHalf == 2, "a wavefront holds 16 or 32 h columns");
+  const int r = lane & 15, gq = lane >> 4;
+  const bool f16 = g.out_dtype != 0;
+  const int inter = g.n >> 1;
+  float* s_amax = (float*)lds;   // [kWavesN][BM]; the ring is free: every wavefront has left the K loop
+  float h[MTW][kHalf][4], amaxv[MTW];
+#pragma unroll
+  for (int mt = 0; mt < MTW; mt++) {
+    float amax = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < kHalf; nt++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        float gv, uv;
+        if (f16) {
+          gv = (float)(_Float16)acc[nt][mt][i];
+          uv = (float)(_Float16)acc[nt + kHalf][mt][i];
+        } else {
+          gv = (float)(__bf16)acc[nt][mt][i];
+          uv = (float)(__bf16)acc[nt + kHalf][mt][i];
+        }
+        float hv = swiglu_f32(gv, uv);
+        hv = f16 ? (float)(_Float16)hv : (float)(__bf16)hv;
+        h[mt][nt][i] = hv;
+        amax = __builtin_fmaxf(amax, __builtin_fabsf(hv));
+      }
+    }
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 16));
+    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 32));
+    amaxv[mt] = amax;
+    if (kPair && gq == 0) s_amax[wn * BM + mw + mt * 16 + r] = amax;
+  }
+  if constexpr (kPair) __syncthreads();
+  uint8_t* sf_e = g.sf_out + (long)g.blockscale_offsets[e] * (inter >> 5);
+  const int cblk = (n0 >> 6) + ((wn * (kRW / 2)) >> 5);   // 32-column block of this wavefront's h columns
+  const int m_pad = (M + 127) & ~127;
+#pragma unroll
+  for (int mt = 0; mt < MTW; mt++) {
+    const int row = mw + mt * 16 + r;
+    const int m = m0 + row;
+    float amax = amaxv[mt];
+    if constexpr (kPair) amax = __builtin_fmaxf(amax, s_amax[(wn ^ 1) * BM + row]);
+    const int code = mx_scale_code(amax);
+    const float inv = mx_scale_inverse(amax, code);
+    if (m < M) {
+      uint8_t* qrow = (uint8_t*)g.q_out + (row_base + m) * (long)inter + (n0 >> 1) + wn * (kRW / 2) + gq * 4;
+#pragma unroll
+      for (int nt = 0; nt < kHalf; nt++) {
+        float y[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) y[i] = __builtin_amdgcn_fmed3f(h[mt][nt][i] * inv, -448.f, 448.f);
+        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+        *(int*)(qrow + nt * 16) = w0;
+      }
+    }
+    if (gq == 0 && (!kPair || (wn & 1) == 0) && m < m_pad) {
+      sf_e[((long)(m >> 7) * (inter >> 7) + (cblk >> 2)) * 512 + (m & 31) * 16 + ((m & 127) >> 5) * 4 + (cblk & 3)] =
+          (uint8_t)(m < M ? code : 0);
+    }
+  }
+  // rows of the expert's last scale tile that lie below this tile: the tile's four scale columns are one dword
+  if (m0 + BM >= M) {
+    for (int m = m0 + BM + (int)threadIdx.x; m < m_pad; m += kThreads) {
+      *(uint32_t*)(sf_e + ((long)(m >> 7) * (inter >> 7) + (n0 >> 8)) * 512 + (m & 31) * 16 + ((m & 127) >> 5) * 4) = 0u;
+    }
+  }
+  if constexpr (kPair) __syncthreads();   // s_amax is ring memory: the next tile's copies must not land before it is read
+}
+
+// FUSE: the weights are a gate_up projection [E, 2I, K] (gate rows first) and the tile's 256 weight rows are 128 gate
+// rows and the matching 128 up rows, interleaved so that every wavefront holds gate and up of the same columns; the
+// epilogue forms silu(gate) * up and quantises it for the down projection (fp8-blockwise: 1x128 blocks with fp32
+// scales, tile_epilogue; mxfp8: 1x32 blocks with E8M0 scales, tile_epilogue_mxq) instead of writing the projection.
 template <int MT, bool MX, bool FUSE>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds) {
-  static_assert(!(MX && FUSE), "the fused SwiGLU epilogue exists for fp8-blockwise only");
+  static_assert(MT == 1 || MT == 2 || MT == 4, "short tiles; 128- and 192-row tiles are gemm_tile_pp / gemm_tile_pp_mx");
   using G = TileGeom<MT, MX>;
   constexpr int MTW = G::MTW, NTW = G::NTW, NBUF = G::kNBuf;
   const int tid = threadIdx.x;
@@ -313,9 +389,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   } else {
     const int kc = K >> 5;
     int blk;
-    if ((wave & 1) == 0) {  // even wavefronts: the two weight scale tiles
+    if ((wave & 1) == 0) {  // even wavefronts: the two weight scale tiles (FUSE: of the gate rows, of the up rows)
       blk = (n0 >> 7) + (lane >> 5);
       if (blk * 128 >= N) blk = n0 >> 7;
+      if constexpr (FUSE) blk = (n0 >> 8) + (lane >> 5) * (N >> 8);
       sc_base = g.sfb + (long)e * N * kc;
     } else {                // odd wavefronts: the token scale tile(s)
       blk = (m0 >> 7) + (lane >> 5);
@@ -387,7 +464,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   constexpr int kScaleOff = G::kABytes + G::kWBytes;
   const float* sb_tab = s_sb + (FUSE ? 0 : (nw >> 7)) * kMaxKB;   // FUSE: table 0 = gate block, table 1 = up block
   // mxfp8: per-lane bases of the scale dwords (weight rows nw + r, token rows mw + r of a tall tile)
-  const int sfw_lane = kScaleOff + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16;
+  // (FUSE: n-tile 0 = gate rows n0/2 + wn*16 + r in the first tile, n-tile 1 the up rows at the same place in the second)
+  const int sfw_lane = FUSE ? kScaleOff + ((wn & 1) * 16 + r) * 16 + (wn >> 1) * 4
+                            : kScaleOff + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16;
   const int sfa_lane = kScaleOff + 1024 + (mw >> 7) * 512 + ((mw & 127) >> 5) * 4 + r * 16;
   const int sa_lane = kScaleOff + (mw + r) * 4;   // fp8-blockwise: float sa of token row mw + r
   const int sa4_lane = kSaChunkOff + (mw + r) * 16;
@@ -403,12 +482,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // the matrix pipe busy, the other group reads its fragments from LDS.
   //   read phase: weight fragments, the first kPre token fragments and all scales -> registers
   //   mfma phase: the MFMAs (+ the fp32 promotion for fp8-blockwise) of the K block
-  // (256-row mxfp8 tiles read only the first token fragment there: their MFMA phase is one hand-scheduled statement
-  // that fetches row tile mt + 1 under the MFMAs of mt and sends the next stage's copies between the MFMAs, see
-  // mx_phase.h.  All eight wavefronts run that phase at the same time, and issued in one burst at the top of the K
-  // block their 72 copies occupied the texture path for ~1000 cycles in which no MFMA ran.)
-  constexpr bool kMx256 = MX && MT == 16;
-  constexpr int kPre = kMx256 ? 1 : MTW < 4 ? MTW : (MTW == 6 ? 6 : 4);
+  constexpr int kPre = MTW;   // every token fragment of a short tile fits in registers
   struct Frags {
     v8i wf[NTW];
     v8i af[kPre];
@@ -430,80 +504,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     }
   };
 
-  // fp8-blockwise tiles of 128 and 192 rows: the copies of K block kb2 into ring slot nbuf, spread between the
-  // fragment reads of slot buf.  A wavefront that issues its copies back to back sits in the queue to the texture
-  // path (one 1 KB copy per ~18 cycles and CU) for as long as the fragment reads then take; interleaved, the two
-  // overlap.  One statement, so that m0 is written once per operand and nothing is scheduled in between; the
-  // fragment halves are read into separate registers that the register allocator places side by side.
-  constexpr bool kInterleave = !MX && (MT == 8 || MT == 12);
-  auto issue_and_read = [&](int kb2, int nbuf, int kb, int buf, Frags& f) {
-    if constexpr (kInterleave) {
-      static_assert(NTW == 4 && G::kWCopies == 4 && kPre == MTW, "interleaved issue: wavefront shape");
-      const uint32_t sbn = lds0 + nbuf * G::kStageBytes;
-      const uint32_t la = sbn + ablk0 * 1024, lw = sbn + G::kABytes + wave * G::kWCopies * 1024;
-      const uint8_t* ap = a_ptr + (long)kb2 * 128;
-      const uint8_t* wp = w_ptr + (long)kb2 * 128;
-      const uint32_t rb = lds0 + buf * G::kStageBytes;
-      const uint32_t wl = rb + wfrag_lo, wh = rb + (wfrag_lo ^ 64), al = rb + afrag_lo, ah = rb + (afrag_lo ^ 64);
-      v4i w0l, w0h, w1l, w1h, w2l, w2h, w3l, w3h, a0l, a0h, a1l, a1h, a2l, a2h, a3l, a3h;
-#define ESMOE_RD(dst, addr, off) "ds_read_b128 %[" #dst "], %[" #addr "] offset:" #off "\n\t"
-#define ESMOE_CP(v, base, off, nt) "global_load_lds_dwordx4 %[" #v "], %[" #base "] offset:" #off nt "\n\t"
-#define ESMOE_OUT(x) [x] "=&v"(x)
-#define ESMOE_FRAG_OUTS                                                                                                     \
-  ESMOE_OUT(w0l), ESMOE_OUT(w0h), ESMOE_OUT(w1l), ESMOE_OUT(w1h), ESMOE_OUT(w2l), ESMOE_OUT(w2h), ESMOE_OUT(w3l), ESMOE_OUT(w3h), \
-  ESMOE_OUT(a0l), ESMOE_OUT(a0h), ESMOE_OUT(a1l), ESMOE_OUT(a1h), ESMOE_OUT(a2l), ESMOE_OUT(a2h), ESMOE_OUT(a3l), ESMOE_OUT(a3h)
-#define ESMOE_COMMON_INS                                                                                                    \
-  [la] "s"(la), [lw] "s"(lw), [ap] "s"(ap), [wp] "s"(wp), [va0] "v"(va[0]), [va1] "v"(va[1]), [vw0] "v"(vw[0]), [vw1] "v"(vw[1]), \
-  [vw2] "v"(vw[2]), [vw3] "v"(vw[3]), [wl] "v"(wl), [wh] "v"(wh), [al] "v"(al), [ah] "v"(ah)
-      if constexpr (MT == 8) {
-#define ESMOE_BODY8(nt)                                                                                                     \
-  "s_mov_b32 m0, %[la]\n\t"                                                                                                 \
-  ESMOE_CP(va0, ap, 0, "") ESMOE_RD(w0l, wl, 0) ESMOE_RD(w0h, wh, 0) ESMOE_RD(a0l, al, 0)                                   \
-  ESMOE_CP(va1, ap, 1024, "") ESMOE_RD(a0h, ah, 0) ESMOE_RD(w1l, wl, 2048) ESMOE_RD(w1h, wh, 2048)                          \
-  "s_mov_b32 m0, %[lw]\n\t"                                                                                                 \
-  ESMOE_CP(vw0, wp, 0, nt) ESMOE_RD(a1l, al, 2048) ESMOE_RD(a1h, ah, 2048) ESMOE_RD(w2l, wl, 4096)                          \
-  ESMOE_CP(vw1, wp, 1024, nt) ESMOE_RD(w2h, wh, 4096) ESMOE_RD(a2l, al, 4096) ESMOE_RD(a2h, ah, 4096)                       \
-  ESMOE_CP(vw2, wp, 2048, nt) ESMOE_RD(w3l, wl, 6144) ESMOE_RD(w3h, wh, 6144) ESMOE_RD(a3l, al, 6144)                       \
-  ESMOE_CP(vw3, wp, 3072, nt) ESMOE_RD(a3h, ah, 6144)                                                                       \
-  "s_waitcnt lgkmcnt(0)"
-        if (w_once) asm volatile(ESMOE_BODY8(" nt") : ESMOE_FRAG_OUTS : ESMOE_COMMON_INS : "memory", "m0");
-        else asm volatile(ESMOE_BODY8("") : ESMOE_FRAG_OUTS : ESMOE_COMMON_INS : "memory", "m0");
-#undef ESMOE_BODY8
-      } else {
-        v4i a4l, a4h, a5l, a5h;
-#define ESMOE_BODY12(nt)                                                                                                    \
-  "s_mov_b32 m0, %[la]\n\t"                                                                                                 \
-  ESMOE_CP(va0, ap, 0, "") ESMOE_RD(w0l, wl, 0) ESMOE_RD(w0h, wh, 0) ESMOE_RD(a0l, al, 0)                                   \
-  ESMOE_CP(va1, ap, 1024, "") ESMOE_RD(a0h, ah, 0) ESMOE_RD(w1l, wl, 2048) ESMOE_RD(w1h, wh, 2048)                          \
-  ESMOE_CP(va2, ap, 2048, "") ESMOE_RD(a1l, al, 2048) ESMOE_RD(a1h, ah, 2048) ESMOE_RD(w2l, wl, 4096)                       \
-  "s_mov_b32 m0, %[lw]\n\t"                                                                                                 \
-  ESMOE_CP(vw0, wp, 0, nt) ESMOE_RD(w2h, wh, 4096) ESMOE_RD(a2l, al, 4096) ESMOE_RD(a2h, ah, 4096)                          \
-  ESMOE_CP(vw1, wp, 1024, nt) ESMOE_RD(w3l, wl, 6144) ESMOE_RD(w3h, wh, 6144) ESMOE_RD(a3l, al, 6144)                       \
-  ESMOE_CP(vw2, wp, 2048, nt) ESMOE_RD(a3h, ah, 6144) ESMOE_RD(a4l, al, 8192) ESMOE_RD(a4h, ah, 8192)                       \
-  ESMOE_CP(vw3, wp, 3072, nt) ESMOE_RD(a5l, al, 10240) ESMOE_RD(a5h, ah, 10240)                                             \
-  "s_waitcnt lgkmcnt(0)"
-        if (w_once)
-          asm volatile(ESMOE_BODY12(" nt") : ESMOE_FRAG_OUTS, ESMOE_OUT(a4l), ESMOE_OUT(a4h), ESMOE_OUT(a5l), ESMOE_OUT(a5h)
-                       : ESMOE_COMMON_INS, [va2] "v"(va[G::kACopies - 1]) : "memory", "m0");
-        else
-          asm volatile(ESMOE_BODY12("") : ESMOE_FRAG_OUTS, ESMOE_OUT(a4l), ESMOE_OUT(a4h), ESMOE_OUT(a5l), ESMOE_OUT(a5h)
-                       : ESMOE_COMMON_INS, [va2] "v"(va[G::kACopies - 1]) : "memory", "m0");
-#undef ESMOE_BODY12
-        f.af[kPre - 2] = join(a4l, a4h);
-        f.af[kPre - 1] = join(a5l, a5h);
-      }
-#undef ESMOE_RD
-#undef ESMOE_CP
-#undef ESMOE_OUT
-#undef ESMOE_FRAG_OUTS
-#undef ESMOE_COMMON_INS
-      f.wf[0] = join(w0l, w0h); f.wf[1] = join(w1l, w1h); f.wf[2] = join(w2l, w2h); f.wf[3] = join(w3l, w3h);
-      f.af[0] = join(a0l, a0h); f.af[1] = join(a1l, a1h); f.af[2] = join(a2l, a2h); f.af[3] = join(a3l, a3h);
-      if (!sa4) dma4(sc_base + (long)kb2 * 4, scoff, sbn + sclds);
-      read_scales_fp8(kb, buf, f);
-    }
-  };
-
   auto read_phase = [&](int kb, int buf, Frags& f) {
     const uint8_t* lb = lds + buf * G::kStageBytes;
 #pragma unroll
@@ -520,24 +520,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
       for (int nt = 0; nt < NTW; nt++) {
         constexpr int kQuarter = NTW == 4 ? 1 : 0;  // NTW = 4: nt/2 selects the 32-row quarter
-        uint32_t d = *(const uint32_t*)(lb + sfw_lane + (nt & 1) * 256 + (kQuarter ? (nt >> 1) * 4 : 0));
+        uint32_t d = *(const uint32_t*)(lb + sfw_lane + (FUSE ? nt * 512 : (nt & 1) * 256 + (kQuarter ? (nt >> 1) * 4 : 0)));
         f.sfw[nt] = (int)(d >> (gq * 8));
       }
 #pragma unroll
       for (int mt = 0; mt < MTW; mt++) {
-        uint32_t d;
-        if constexpr (MT == 16) {
-          // 256-row tiles start on a 128-row boundary and a wavefront's rows on a multiple of 128: row tile mt adds
-          // compile-time offsets
-          d = *(const uint32_t*)(lb + sfa_lane + (mt >> 3) * 512 + (mt & 1) * 256 + ((mt & 7) >> 1) * 4);
-        } else if constexpr (MT == 12 || MT == 8) {
-          // 128- and 192-row tiles may start in the middle of a scale tile (full tiles of 192 rows)
-          int ml = (m0 & 127) + mw + mt * 16 + r;
-          d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4);
-        } else {
-          int ml = (m0 & 127) + mt * 16 + r;  // token row inside its 128-row scale tile
-          d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml & 31) * 16 + (ml >> 5) * 4);
-        }
+        // token row inside its 128-row scale tile (a short tile starts on a multiple of 64 rows and never crosses one)
+        const int ml = (m0 & 127) + mt * 16 + r;
+        const uint32_t d = *(const uint32_t*)(lb + kScaleOff + 1024 + (ml & 31) * 16 + (ml >> 5) * 4);
         f.sfa[mt] = (int)(d >> (gq * 8));
       }
     } else {
@@ -545,21 +535,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     }
   };
 
-  // 256-row mxfp8 tiles: the whole phase is the statement of mx_phase.h.
-  // One statement for every K block, so that the accumulators keep their registers around the loop: past the last
-  // K block that has a stage to fetch, the copies fetch the last K block once more into the slot that is free anyway.
-  auto mfma_phase_mx = [&](int buf, const Frags& f, int kb2, int slot) {
-    if constexpr (kMx256) {
-      const uint32_t rb = lds0 + buf * G::kStageBytes;
-      const uint32_t al = rb + afrag_lo, ah = rb + (afrag_lo ^ 64);
-      const uint32_t sbn = lds0 + slot * G::kStageBytes;
-      const uint32_t la = sbn + ablk0 * 1024, lw = sbn + G::kABytes + wave * G::kWCopies * 1024, ls = sbn + sclds;
-      const uint8_t* ap = a_ptr + (long)kb2 * 128;
-      const uint8_t* wp = w_ptr + (long)kb2 * 128;
-      const uint8_t* sp = sc_base + (long)kb2 * 512;
-      asm volatile(ESMOE_MX256_PHASE : ESMOE_MX256_OUTS : ESMOE_MX256_INS : ESMOE_MX256_CLOBBERS);
-    }
-  };
   // fp8-blockwise with all fragments in registers: MFMAs and promotions form one scheduling region in which
   // the four v_fmac of MFMA j - 3 follow MFMA j, so the vector ALU works in the shadow of the matrix pipe
   // and no promotion waits on the MFMA it has just been issued behind.  Taller tiles (fragments read from
@@ -716,13 +691,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       chunk_age = 0;
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (kInterleave && more) {
-      issue_and_read(kb + NBUF - 1, nbuf, kb, buf, f);
-    } else {
-      if (more) { if constexpr (kSplitIssue) issue_a(kb + NBUF - 1, nbuf); else if constexpr (!kMx256) issue(kb + NBUF - 1, nbuf); }
-      __builtin_amdgcn_sched_barrier(0);
-      read_phase(kb, buf, f);
-    }
+    if (more) { if constexpr (kSplitIssue) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
+    __builtin_amdgcn_sched_barrier(0);
+    read_phase(kb, buf, f);
     __builtin_amdgcn_sched_barrier(0);
     if (grp == 1) wait_stage(more, chunk_age < NBUF - 2);
     if constexpr (kPP) block_barrier();
@@ -731,8 +702,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       else if (kb + NBUF < KB) issue_w(kb + NBUF, buf);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (kMx256) mfma_phase_mx(buf, f, more ? kb + NBUF - 1 : KB - 1, nbuf);
-    else mfma_phase(buf, f);
+    mfma_phase(buf, f);
     __builtin_amdgcn_sched_barrier(0);
     if (grp == 0) wait_stage(more, chunk_age < NBUF - 2);
     chunk_age++;
@@ -742,7 +712,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   }
   if (kPP && grp == 0) block_barrier();
 
-  tile_epilogue<G::BM, MTW, NTW, G::kWavesN, FUSE>(g, acc, M, m0, n0, row_base, mw, nw, wn, lane, wave_active, lds);
+  if constexpr (MX && FUSE) tile_epilogue_mxq<G::BM, MTW, NTW, G::kWavesN>(g, acc, e, M, m0, n0, row_base, mw, wn, lane, lds);
+  else tile_epilogue<G::BM, MTW, NTW, G::kWavesN, FUSE>(g, acc, M, m0, n0, row_base, mw, nw, wn, lane, wave_active, lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -930,7 +901,7 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
 //         1 KB spare, the target of the scale copies of the wavefronts that have no scale tile to fetch
 // A tile may start in the middle of a 128-row scale tile (full tiles are 192 rows): a lane finds the scale dword of
 // its row from the row's position inside the two tiles that were fetched for its group.
-template <int MT>
+template <int MT, bool FUSE>
 __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds,
                                                 uint32_t* timeline = nullptr) {
   static_assert(MT == 8 || MT == 12, "hand-scheduled K block: 128- and 192-row tiles");
@@ -965,11 +936,18 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int blk = wave * 4 + i;
-    const int row = (n0 + blk * 8 < N ? blk : i) * 8;
+    int row;
+    if constexpr (FUSE) {   // 32 gate rows, then the matching 32 up rows, per wavefront column (see gemm_tile_pp)
+      constexpr int kRW = NTW * 16, kBlocks = kRW / 8, kHalfBlocks = kBlocks / 2;
+      const int wcol = blk / kBlocks, within = blk % kBlocks;
+      row = (within / kHalfBlocks) * (N >> 1) + (n0 >> 1) + wcol * (kRW / 2) + (within % kHalfBlocks) * 8;
+    } else {
+      row = (n0 + blk * 8 < N ? blk : i) * 8;
+    }
     vw[i] = (uint32_t)(row + crow) * (uint32_t)K + (swz(blk * 8 + crow, cslot) << 4) + kBias - i * 1024;
   }
   const uint8_t* a_ptr = (const uint8_t*)g.a + (row_base + m0) * K - kBias;
-  const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + n0) * K - kBias;
+  const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + (FUSE ? 0 : n0)) * K - kBias;
   const uint32_t t_dst = lds0 + kTBase + grp * 2 * kTSlot + wj * kTCopies * 1024;   // + slot * kTSlot
   const uint32_t w_dst = lds0 + wave * 4096;                                        // + slot * kWSlot
   // scale copies, one per wavefront and K block: wavefront 0 the weight scale tiles (with the weight stage),
@@ -981,6 +959,7 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
   if (s_role == 0) {
     int blk = (n0 >> 7) + (lane >> 5);
     if (blk * 128 >= N) blk = n0 >> 7;
+    if constexpr (FUSE) blk = (n0 >> 8) + (lane >> 5) * (N >> 8);   // scale tile of the gate rows, of the up rows
     s_ptr = g.sfb + (long)e * N * kc;
     vs = (uint32_t)blk * (uint32_t)KB * 512 + (lane & 31) * 16;
     s_dst = lds0 + kBN * 128;                // + slot * kWSlot
@@ -1008,8 +987,11 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
   // ---- fragment and scale read plan -------------------------------------------------------------------------
   const uint32_t wfrag = lds0 + (nw + r) * 128 + swz(r, gq) * 16;                       // + slot * kWSlot
   const uint32_t afrag = lds0 + kTBase + grp * 2 * kTSlot + r * 128 + swz(r, gq) * 16;  // + slot * kTSlot
-  // weight scale dword of row nw + nt*16 + r: n-tile nt at + (nt & 1)*256 + (nt >> 1)*4
-  const uint32_t sfw_rd = lds0 + kBN * 128 + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16;
+  // weight scale dword of row nw + nt*16 + r: n-tile nt at + (nt & 1)*256 + (nt >> 1)*4.  FUSE: the wavefront's gate
+  // rows are rows wj*32 + nt*16 + r of the first tile (n-tiles 0, 1), its up rows the same rows of the second (2, 3):
+  // n-tile nt at + (nt & 1)*256 + (nt >> 1)*512
+  const uint32_t sfw_rd = FUSE ? lds0 + kBN * 128 + r * 16 + wj * 4
+                               : lds0 + kBN * 128 + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16;
   uint32_t sfa_rd[MTW];
 #pragma unroll
   for (int mt = 0; mt < MTW; mt++) {
@@ -1056,7 +1038,9 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
       uint32_t sfal[MTW];
 #pragma unroll
       for (int mt = 0; mt < MTW; mt++) sfal[mt] = sfa_rd[mt] + tslot * kTSlot;
-      if constexpr (MT == 12) ESMOE_PP_STMT(ESMOE_PPX12);
+      if constexpr (MT == 12 && FUSE) ESMOE_PP_STMT(ESMOE_PPX12F);
+      else if constexpr (MT == 12) ESMOE_PP_STMT(ESMOE_PPX12);
+      else if constexpr (FUSE) ESMOE_PP_STMT(ESMOE_PPX8F);
       else ESMOE_PP_STMT(ESMOE_PPX8);
       tslot ^= 1;
       wslot = wslot == 2 ? 0 : wslot + 1;
@@ -1073,7 +1057,8 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
   wait_vmcnt<0>();
   if (grp == 0) block_barrier();
   block_barrier();
-  tile_epilogue<BM, MTW, NTW, 4, false>(g, acc, M, m0, n0, row_base, mw, nw, wj, lane, wave_active, lds);
+  if constexpr (FUSE) tile_epilogue_mxq<BM, MTW, NTW, 4>(g, acc, e, M, m0, n0, row_base, mw, wj, lane, lds);
+  else tile_epilogue<BM, MTW, NTW, 4, false>(g, acc, M, m0, n0, row_base, mw, nw, wj, lane, wave_active, lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1250,10 +1235,10 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     bool hand_scheduled = false;
     if constexpr (MX) {
       if ((ESMOE_PPX_HEIGHTS & 2) && t.mt == 12) {
-        gemm_tile_pp_mx<12>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        gemm_tile_pp_mx<12, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
         hand_scheduled = true;
       } else if ((ESMOE_PPX_HEIGHTS & 1) && t.mt == 8) {
-        gemm_tile_pp_mx<8>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        gemm_tile_pp_mx<8, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
         hand_scheduled = true;
       }
     }
@@ -1327,7 +1312,9 @@ extern "C" int esmoe_launch_grouped_gemm(const esmoe::GemmArgs* args, int mx, in
                      args->policy, args->ws);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return (int)err;
-  if (mx)
+  if (mx && args->q_out)
+    hipLaunchKernelGGL((grouped_gemm_kernel<true, true>), dim3(grid), dim3(kThreads), 0, stream, *args);
+  else if (mx)
     hipLaunchKernelGGL((grouped_gemm_kernel<true, false>), dim3(grid), dim3(kThreads), 0, stream, *args);
   else if (args->q_out)
     hipLaunchKernelGGL((grouped_gemm_kernel<false, true>), dim3(grid), dim3(kThreads), 0, stream, *args);

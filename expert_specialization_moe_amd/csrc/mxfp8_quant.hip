@@ -25,6 +25,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "mx_scale.h"
 #include "swiglu.h"
 
 namespace esmoe {
@@ -51,14 +52,6 @@ __device__ __forceinline__ void unpack8(v4i raw, float* x) {
       x[2 * i + 1] = __builtin_bit_cast(float, w & 0xffff0000u);
     }
   }
-}
-
-// E8M0 code of the smallest power of two >= amax / 448 (amax >= 0, finite).
-__device__ __forceinline__ int mx_scale_code(float amax) {
-  uint32_t bits = __builtin_bit_cast(uint32_t, amax);
-  int code = (int)((bits >> 23) & 0xff) - 8 + ((bits & 0x7fffffu) > 0x600000u ? 1 : 0);
-  code = code < 0 ? 0 : (code > 254 ? 254 : code);
-  return amax == 0.f ? 0 : code;
 }
 
 template <bool FP16>
@@ -137,7 +130,7 @@ __global__ void __launch_bounds__(quant_threads<SWIGLU>()) __attribute__((amdgpu
     amax = __builtin_fmaxf(amax, __shfl_xor(amax, 1));
     amax = __builtin_fmaxf(amax, __shfl_xor(amax, 2));
     const int code = mx_scale_code(amax);
-    const float inv = amax == 0.f ? 0.f : __builtin_bit_cast(float, (uint32_t)(254 - code) << 23);
+    const float inv = mx_scale_inverse(amax, code);
     float y[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) y[i] = __builtin_amdgcn_fmed3f(x[i] * inv, -448.f, 448.f);
