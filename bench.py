@@ -52,8 +52,12 @@ def parse():
                          "swiglu_quant: fused SwiGLU + 1x128 quantisation of the workload's [rows, N] output")
     ap.add_argument("--force-bm", type=int, default=0, help="single M-tile shape for every expert (0 = device schedule)")
     ap.add_argument("--fuse-swiglu", action="store_true",
-                    help="gemm op, fp8-blockwise configs: the projection with the fused SwiGLU + 1x128 quantisation epilogue "
-                         "(the workload's N is read as 2 * inter); the output bytes counted are the e4m3 + scale bytes")
+                    help="gemm op: the projection with the fused SwiGLU + re-quantisation epilogue (1x128 fp32 scales for the "
+                         "fp8-blockwise configs, 1x32 E8M0 scales for c4; the workload's N is read as 2 * inter); the output "
+                         "bytes counted are the e4m3 + scale bytes")
+    ap.add_argument("--single-tile-sweep", action="store_true",
+                    help="gemm op: after the timed region also time the same kernel with every single tile height forced "
+                         "(16 .. 192 rows) and report the best one and its ratio to the device schedule's time")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="after the timed region also run three 1 GiB device copies (a kernel of known traffic, for "
@@ -421,29 +425,55 @@ def main():
     def vp(t):
         return ctypes.c_void_p(t.data_ptr())
 
-    if args.fuse_swiglu:
-        assert not mx and n % 256 == 0, "--fuse-swiglu needs an fp8-blockwise config with N a multiple of 256"
-        q_f = torch.empty((total, n // 2), dtype=torch.uint8, device=dev)
-        sc_f = torch.empty((total, n // 256), dtype=torch.float32, device=dev)
-
-        def step():
-            es.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(q_f, sc_f, ops["a"], ops["b"], ops["scales_a"], ops["scales_b"],
-                                                               ops["problem_sizes"], ops["expert_offsets"], ops["workspace"])
-    elif args.force_bm:
+    def forced_step(force_bm):
         # single-tile-shape baseline: same kernel, one M-tile height for every expert (C ABI only)
         def step():
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             if mx:
                 rc = lib.esmoe_mxfp8_grouped_mm(vp(ops["output"]), 0, vp(ops["a"]), vp(ops["b_phys"]), vp(ops["sfa"]),
                                                 vp(ops["sfb_phys"]), vp(ops["problem_sizes"]), vp(ops["expert_offsets"]),
-                                                vp(ops["blockscale_offsets"]), e, total, n, k, args.force_bm, vp(ws),
+                                                vp(ops["blockscale_offsets"]), e, total, n, k, force_bm, vp(ws),
                                                 ws_bytes, stream)
             else:
                 rc = lib.esmoe_fp8_blockwise_grouped_mm(vp(ops["output"]), 0, vp(ops["a"]), vp(ops["b_phys"]),
                                                         vp(ops["scales_a"]), vp(ops["scales_b_phys"]),
                                                         vp(ops["problem_sizes"]), vp(ops["expert_offsets"]), e, total, n,
-                                                        k, args.force_bm, vp(ws), ws_bytes, stream)
+                                                        k, force_bm, vp(ws), ws_bytes, stream)
             assert rc == 0, _native.last_error()
+        return step
+
+    def time_steps(fn, warmup, steps):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(steps):
+            fn()
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / steps
+
+    if args.fuse_swiglu:
+        assert n % 256 == 0, "--fuse-swiglu needs N a multiple of 256"
+        q_f = torch.empty((total, n // 2), dtype=torch.uint8, device=dev)
+        if mx:
+            sf_f = torch.empty((ops["sfa"].shape[0], n // 64), dtype=torch.uint8, device=dev)
+
+            def step():
+                es.es_mxfp8_blockscaled_grouped_mm_swiglu_quant(q_f, sf_f, ops["a"], ops["b"], ops["sfa"], ops["sfb"],
+                                                                ops["problem_sizes"], ops["expert_offsets"],
+                                                                ops["blockscale_offsets"])
+        else:
+            sc_f = torch.empty((total, n // 256), dtype=torch.float32, device=dev)
+
+            def step():
+                es.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(q_f, sc_f, ops["a"], ops["b"], ops["scales_a"],
+                                                                   ops["scales_b"], ops["problem_sizes"],
+                                                                   ops["expert_offsets"], ops["workspace"])
+    elif args.force_bm:
+        step = forced_step(args.force_bm)
     elif mx:
         def step():
             es.es_sm100_mxfp8_blockscaled_grouped_mm(ops["output"], ops["a"], ops["b"], ops["sfa"], ops["sfb"],
@@ -473,7 +503,8 @@ def main():
     nbytes = W.gemm_bytes(prob.rows, n, k, prob.kind)
     t_roof = W.gemm_roofline_seconds(prob.rows, n, k, prob.kind)
     if args.fuse_swiglu:
-        nbytes += total * (n / 2 + 4.0 * n / 256) - 2.0 * n * total     # e4m3 + scales written instead of bf16
+        # e4m3 + scales (fp32 per 128 columns, or one byte per 32) written instead of bf16
+        nbytes += total * (n / 2 + (n / 64 if mx else 4.0 * n / 256)) - 2.0 * n * total
         t_roof = max(flops / W.FP8_FLOPS_PER_S, nbytes / W.HBM_BYTES_PER_S)
     t = ms_per_step * 1e-3
     hbm_bound = nbytes / W.HBM_BYTES_PER_S >= flops / W.FP8_FLOPS_PER_S
@@ -496,6 +527,13 @@ def main():
                    "force_bm": args.force_bm, "fuse_swiglu": bool(args.fuse_swiglu), "routing_meta": prob.meta},
         "roofline": roof, "wall_ms_per_step": wall * 1e3 / args.steps,
     }
+    if args.single_tile_sweep:
+        # the best any single tile height does on this workload, on the same kernel and the same operands
+        sweep = {bm: time_steps(forced_step(bm), args.warmup, args.steps) * 1e3 for bm in (16, 32, 64, 128, 192)}
+        best = min(sweep, key=sweep.get)
+        out["single_tile_sweep"] = {"us_by_tile_rows": sweep, "best_single_tile_rows": best,
+                                    "best_single_tile_us": sweep[best], "device_schedule_us": ms_per_step * 1e3,
+                                    "ratio": sweep[best] / (ms_per_step * 1e3)}
     if args.calibration_copy:
         calibration_copy()
     if not args.no_cpu_baseline:

@@ -20,6 +20,7 @@ from .ops import (  # noqa: F401
     es_swiglu_mxfp8_grouped_quant,
     es_mxfp8_quant_weight,
     es_fp8_blockwise_scaled_grouped_mm_swiglu_quant,
+    es_mxfp8_blockscaled_grouped_mm_swiglu_quant,
 )
 
 __all__ = [
@@ -34,4 +35,5 @@ __all__ = [
     "es_swiglu_mxfp8_grouped_quant",
     "es_mxfp8_quant_weight",
     "es_fp8_blockwise_scaled_grouped_mm_swiglu_quant",
+    "es_mxfp8_blockscaled_grouped_mm_swiglu_quant",
 ]

@@ -45,6 +45,9 @@ lib.esmoe_mxfp8_grouped_quant.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, 
 lib.esmoe_fp8_blockwise_grouped_mm_swiglu_quant.restype = _i
 lib.esmoe_fp8_blockwise_grouped_mm_swiglu_quant.argtypes = [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp,
                                                             ctypes.c_size_t, _vp]
+lib.esmoe_mxfp8_grouped_mm_swiglu_quant.restype = _i
+lib.esmoe_mxfp8_grouped_mm_swiglu_quant.argtypes = [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp,
+                                                    ctypes.c_size_t, _vp]
 lib.esmoe_swiglu_mxfp8_grouped_quant.restype = _i
 lib.esmoe_swiglu_mxfp8_grouped_quant.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]
 lib.esmoe_mxfp8_quant_weight.restype = _i

@@ -254,6 +254,32 @@ int esmoe_mxfp8_grouped_mm(void* d, int out_dtype, const void* a, const void* b,
   return launch_gemm(g, 1, force_bm, stream);
 }
 
+int esmoe_mxfp8_grouped_mm_swiglu_quant(void* q, uint8_t* sf, int mid_dtype, const void* a, const void* b,
+                                        const uint8_t* sfa, const uint8_t* sfb, const int32_t* problem_sizes,
+                                        const int32_t* expert_offsets, const int32_t* blockscale_offsets,
+                                        int num_experts, int total_rows, int sf_rows, int n, int k, int force_bm,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int rc = check_common(q, a, b, problem_sizes, expert_offsets, num_experts, total_rows, n, k, force_bm, workspace,
+                        workspace_bytes, mid_dtype);
+  if (rc) return rc;
+  if (!sfa || !sfb || !sf || !blockscale_offsets) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null scale pointer");
+  if ((uintptr_t)sfa % 4 || (uintptr_t)sfb % 4 || (uintptr_t)sf % 4 || (uintptr_t)q % 4)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "sfa, sfb, sf and q must be 4-byte aligned");
+  if (n % 256) return fail(ESMOE_ERR_INVALID_ARGUMENT, "n = 2 * inter with inter a multiple of 128, got n = %d", n);
+  // every expert's scale rows are padded to 128, so sf holds at least the row total rounded up
+  if (sf_rows % 128 || sf_rows < (total_rows + 127) / 128 * 128)
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "sf_rows must be a multiple of 128 and >= total_rows rounded up to 128, got %d",
+                sf_rows);
+  esmoe::GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.b = b; g.sfa = sfa; g.sfb = sfb; g.q_out = q; g.sf_out = sf;
+  g.problem_sizes = problem_sizes; g.expert_offsets = expert_offsets; g.blockscale_offsets = blockscale_offsets;
+  g.ws = (int32_t*)workspace;
+  g.num_experts = num_experts; g.total_rows = total_rows; g.n = n; g.k = k; g.out_dtype = mid_dtype;
+  return launch_gemm(g, 1, force_bm, stream);
+}
+
 namespace {
 int grouped_quant_common(const void* in, int in_dtype, const int32_t* problem_sizes, const int32_t* expert_offsets,
                          const int32_t* blockscale_offsets, void* q, uint8_t* sf, int num_experts, int total_rows,

@@ -226,6 +226,65 @@ void es_sm100_mxfp8_blockscaled_grouped_mm(const torch::Tensor& a, const torch::
   check_rc(rc, "es_sm100_mxfp8_blockscaled_grouped_mm");
 }
 
+// The mxfp8 gate_up projection with SwiGLU and the 1x32 E8M0 re-quantisation fused into its epilogue (no counterpart
+// in the reference).  Operand layouts as es_sm100_mxfp8_blockscaled_grouped_mm with n = 2 * inter; the outputs are what
+// es_sm100_mxfp8_blockscaled_grouped_quant would write for a (rows, inter) input.
+void es_mxfp8_blockscaled_grouped_mm_swiglu_quant(torch::Tensor& quant_output, torch::Tensor& scale_factor,
+                                                  const torch::Tensor& a, const torch::Tensor& b,
+                                                  const torch::Tensor& sfa, const torch::Tensor& sfb,
+                                                  const torch::Tensor& problem_sizes, const torch::Tensor& expert_offsets,
+                                                  const torch::Tensor& blockscale_offsets, bool mid_dtype_bf16) {
+  TORCH_CHECK(problem_sizes.dim() == 2 && problem_sizes.size(1) == 3, "problem_sizes must have shape (num_experts, 3)");
+  const int64_t num_experts = problem_sizes.size(0);
+  TORCH_CHECK(expert_offsets.dim() == 1 && expert_offsets.size(0) == num_experts && blockscale_offsets.dim() == 1 &&
+                  blockscale_offsets.size(0) == num_experts,
+              "expert_offsets and blockscale_offsets must be 1D and have size equal to the number of experts");
+  TORCH_CHECK(problem_sizes.dtype() == torch::kInt32 && expert_offsets.dtype() == torch::kInt32 &&
+                  blockscale_offsets.dtype() == torch::kInt32,
+              "problem_sizes, expert_offsets and blockscale_offsets must be int32");
+  TORCH_CHECK(num_experts >= 1 && num_experts <= ESMOE_MAX_EXPERTS, "Number of experts cannot exceed 1024");
+  TORCH_CHECK(a.dim() == 2 && a.stride(1) == 1 && a.stride(0) == a.size(1), "a must be a packed row-major (rows, k) tensor");
+  TORCH_CHECK(b.dim() == 3 && b.size(0) == num_experts, "b must be a (num_experts, k, n) tensor");
+  TORCH_CHECK(b.stride(1) == 1 && b.stride(2) == b.size(1) && b.stride(0) == b.size(1) * b.size(2),
+              "b must be the column-major (num_experts, k, n) view of a packed (num_experts, n, k) tensor");
+  TORCH_CHECK(a.element_size() == 1 && b.element_size() == 1, "a and b must be 1-byte e4m3 tensors");
+  const int64_t total_rows = a.size(0), k = a.size(1), n = b.size(2);
+  TORCH_CHECK(b.size(1) == k, "a and b disagree on k");
+  TORCH_CHECK(k % 128 == 0 && n % 256 == 0, "k must be a multiple of 128 and n = 2 * inter a multiple of 256");
+  const int64_t inter = n / 2;
+  TORCH_CHECK(quant_output.is_contiguous() && quant_output.element_size() == 1 && quant_output.numel() == total_rows * inter,
+              "quant_output must be a contiguous 1-byte tensor of rows * n / 2 elements");
+  TORCH_CHECK(scale_factor.is_contiguous() && scale_factor.element_size() == 1,
+              "scale_factor must be a contiguous 1-byte tensor");
+  const int64_t sf_rows = (scale_factor.numel() / (inter / 32)) / 128 * 128;
+  TORCH_CHECK(sf_rows >= (total_rows + 127) / 128 * 128,
+              "scale_factor is smaller than the rows rounded up to 128 times n / 64 bytes");
+  TORCH_CHECK(sfa.element_size() == 1 && sfb.element_size() == 1, "scale factors must be 1-byte E8M0");
+  TORCH_CHECK(sfb.numel() >= num_experts * n * (k / 32), "sfb is smaller than num_experts * n * k / 32 bytes");
+  TORCH_CHECK(sfa.numel() >= (total_rows + 127) / 128 * 128 * (k / 32),
+              "sfa is smaller than the rows rounded up to 128 times k / 32 bytes");
+  TORCH_CHECK(total_rows < (int64_t(1) << 31) && sf_rows < (int64_t(1) << 31) && n < (int64_t(1) << 31) &&
+                  k < (int64_t(1) << 31),
+              "tensor too large");
+  require_device(a, "es_mxfp8_blockscaled_grouped_mm_swiglu_quant");
+  for (const torch::Tensor* t : {(const torch::Tensor*)&quant_output, (const torch::Tensor*)&scale_factor, &b, &sfa, &sfb,
+                                 &problem_sizes, &expert_offsets, &blockscale_offsets}) {
+    TORCH_CHECK(t->device() == a.device(), "all tensors must be on the same device");
+  }
+  TORCH_CHECK(problem_sizes.is_contiguous() && expert_offsets.is_contiguous() && blockscale_offsets.is_contiguous(),
+              "metadata tensors must be contiguous");
+  if (total_rows == 0) return;
+  c10::DeviceGuard guard(a.device());
+  torch::Tensor ws = schedule_scratch(nullptr, num_experts, a);
+  int rc = esmoe_mxfp8_grouped_mm_swiglu_quant(
+      quant_output.data_ptr(), (uint8_t*)scale_factor.data_ptr(), mid_dtype_bf16 ? ESMOE_OUT_BF16 : ESMOE_OUT_FP16,
+      a.data_ptr(), b.data_ptr(), (const uint8_t*)sfa.data_ptr(), (const uint8_t*)sfb.data_ptr(),
+      problem_sizes.data_ptr<int32_t>(), expert_offsets.data_ptr<int32_t>(), blockscale_offsets.data_ptr<int32_t>(),
+      (int)num_experts, (int)total_rows, (int)sf_rows, (int)n, (int)k, /*force_bm=*/0, ws.data_ptr(), ws.nbytes(),
+      current_stream(a));
+  check_rc(rc, "es_mxfp8_blockscaled_grouped_mm_swiglu_quant");
+}
+
 void es_sm100_mxfp8_blockscaled_grouped_quant(const torch::Tensor& input, const torch::Tensor& problem_sizes,
                                               const torch::Tensor& expert_offsets,
                                               const torch::Tensor& blockscale_offsets, torch::Tensor& quant_output,
@@ -479,6 +538,9 @@ TORCH_LIBRARY(expert_specialization, m) {
   m.def("es_fp8_quant_weight_128x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def("es_swiglu_quant_1x128(Tensor input, Tensor quant_output, Tensor scales) -> ()");
   m.def(
+      "es_mxfp8_blockscaled_grouped_mm_swiglu_quant(Tensor quant_output, Tensor scale_factor, Tensor a, Tensor b, Tensor "
+      "sfa, Tensor sfb, Tensor problem_sizes, Tensor expert_offsets, Tensor blockscale_offsets, bool mid_dtype_bf16) -> ()");
+  m.def(
       "es_swiglu_mxfp8_grouped_quant(Tensor input, Tensor problem_sizes, Tensor expert_offsets, Tensor "
       "blockscale_offsets, Tensor quant_output, Tensor scale_factor) -> ()");
   m.def("es_mxfp8_quant_weight(Tensor input, Tensor quant_output, Tensor scale_factor) -> ()");
@@ -494,6 +556,7 @@ TORCH_LIBRARY_IMPL(expert_specialization, CUDA, m) {
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
   m.impl("es_swiglu_quant_1x128", &es_swiglu_quant_1x128);
+  m.impl("es_mxfp8_blockscaled_grouped_mm_swiglu_quant", &es_mxfp8_blockscaled_grouped_mm_swiglu_quant);
   m.impl("es_swiglu_mxfp8_grouped_quant", &es_swiglu_mxfp8_grouped_quant);
   m.impl("es_mxfp8_quant_weight", &es_mxfp8_quant_weight);
   m.impl("es_route_metadata", &es_route_metadata);
@@ -509,6 +572,7 @@ TORCH_LIBRARY_IMPL(expert_specialization, CPU, m) {
   m.impl("es_fp8_quant_act_1x128", &es_fp8_quant_act_1x128);
   m.impl("es_fp8_quant_weight_128x128", &es_fp8_quant_weight_128x128);
   m.impl("es_swiglu_quant_1x128", &es_swiglu_quant_1x128);
+  m.impl("es_mxfp8_blockscaled_grouped_mm_swiglu_quant", &es_mxfp8_blockscaled_grouped_mm_swiglu_quant);
   m.impl("es_swiglu_mxfp8_grouped_quant", &es_swiglu_mxfp8_grouped_quant);
   m.impl("es_mxfp8_quant_weight", &es_mxfp8_quant_weight);
   m.impl("es_route_metadata", &es_route_metadata);

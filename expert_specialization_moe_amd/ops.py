@@ -118,3 +118,15 @@ def es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(quant_output, scales_out, a,
     _ns.es_fp8_blockwise_scaled_grouped_mm_swiglu_quant.default(quant_output, scales_out, a, b, scales_a, scales_b,
                                                                 problem_sizes, expert_offsets, workspace,
                                                                 mid_dtype == torch.bfloat16)
+
+
+def es_mxfp8_blockscaled_grouped_mm_swiglu_quant(quant_output, scale_factor, a, b, sfa, sfb, problem_sizes, expert_offsets,
+                                                 blockscale_offsets, mid_dtype=torch.bfloat16):
+    """gate_up projection + SwiGLU + 1x32 E8M0 re-quantisation in one kernel: writes the down projection's ``a``
+    (e4m3 bytes [M, I]) and ``sfa`` (swizzled scale tiles for K = I, in the layout of
+    es_sm100_mxfp8_blockscaled_grouped_quant) where ``b`` is the (E, K, 2I) view of gate_up weights [E, 2I, K]
+    (gate rows first).  Same bytes as es_sm100_mxfp8_blockscaled_grouped_mm (output of ``mid_dtype``) followed by
+    es_swiglu_mxfp8_grouped_quant; no counterpart in the reference."""
+    _ns.es_mxfp8_blockscaled_grouped_mm_swiglu_quant.default(quant_output, scale_factor, a, b, sfa, sfb, problem_sizes,
+                                                             expert_offsets, blockscale_offsets,
+                                                             mid_dtype == torch.bfloat16)

@@ -115,6 +115,27 @@ int esmoe_fp8_blockwise_grouped_mm_swiglu_quant(void* q, float* scales, int mid_
                                                 void* stream);
 
 /*
+ * MXFP8 grouped GEMM of a gate_up projection with the SwiGLU and the 1x32 E8M0 re-quantisation fused into its
+ * epilogue: produces the `a` / `sfa` operands of the down projection directly, without the bf16 [total_rows, n]
+ * intermediate.  No counterpart in the reference (its callers run projection, activation and quantisation as
+ * separate steps); the arithmetic is that of esmoe_mxfp8_grouped_mm followed by esmoe_swiglu_mxfp8_grouped_quant,
+ * step for step, so the two routes give the same bytes.
+ *
+ *   b [E, n, K] with n = 2 * inter: weight rows [0, inter) are the gate, [inter, 2 * inter) the up projection
+ *   (inter % 128 == 0); sfb as for esmoe_mxfp8_grouped_mm.
+ *   q [total_rows, inter] e4m3 bytes;  sf: `sf_rows` rows of inter/32 scale bytes in the layout
+ *   esmoe_mxfp8_grouped_quant writes for K = inter (expert e at byte blockscale_offsets[e] * inter/32, padding
+ *   rows of an expert's last 128-row tile written as 0); sf_rows as there.
+ *   mid_dtype: ESMOE_OUT_BF16 / ESMOE_OUT_FP16, the type the projection and the activation are rounded to on the way.
+ * The other arguments are those of esmoe_mxfp8_grouped_mm.
+ */
+int esmoe_mxfp8_grouped_mm_swiglu_quant(void* q, uint8_t* sf, int mid_dtype, const void* a, const void* b,
+                                        const uint8_t* sfa, const uint8_t* sfb, const int32_t* problem_sizes,
+                                        const int32_t* expert_offsets, const int32_t* blockscale_offsets,
+                                        int num_experts, int total_rows, int sf_rows, int n, int k, int force_bm,
+                                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * MXFP8 grouped quantisation: bf16/fp16 rows -> e4m3 bytes + swizzled E8M0 scales.
  * Replaces es_sm100_mxfp8_blockscaled_grouped_quant
  *   (expert_specialization/csrc/cuda/es_sm100_mxfp8_blockscaled_group_quant.cu:5-39,
