@@ -20,10 +20,10 @@ import torch
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "gemm"): 1.386e9,     # FETCH 650,433.5 x 2.000 KiB + WRITE 52,857.2 x 1.000 KiB
-    ("c2", "gemm"): 4.473e8,     # FETCH 216,577.7 x 2.000 KiB + WRITE 3,627.4 x 1.000 KiB
-    ("c4", "gemm"): 1.270e9,     # FETCH 586,832.1 x 2.000 KiB + WRITE 66,473.2 x 1.000 KiB
-    ("c4", "quant"): 1.786e8,    # FETCH 57,399.6 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
+    ("c1", "gemm"): 1.557e9,     # FETCH 733,580.0 x 2.000 KiB + WRITE 53,274.6 x 1.000 KiB
+    ("c2", "gemm"): 4.486e8,     # FETCH 217,244.9 x 2.000 KiB + WRITE 3,627.6 x 1.000 KiB
+    ("c4", "gemm"): 1.458e9,     # FETCH 678,663.1 x 2.000 KiB + WRITE 66,279.4 x 1.000 KiB
+    ("c4", "quant"): 1.786e8,    # FETCH 57,400.1 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
 }
 
 

@@ -161,6 +161,10 @@ def ablated(lines):
             continue
         if "vmwait" in ABLATE and l.startswith("s_waitcnt vmcnt"):
             continue
+        if "relaxw" in ABLATE and l.startswith("s_waitcnt vmcnt("):
+            n = int(l.split("(")[1].split(")")[0])
+            if n > 4:
+                l = l.replace(f"vmcnt({n})", f"vmcnt({n + 4})")
         out.append(l)
     return out
 
