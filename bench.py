@@ -20,11 +20,23 @@ import torch
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "gemm"): 1.557e9,     # FETCH 733,580.0 x 2.000 KiB + WRITE 53,274.6 x 1.000 KiB
-    ("c2", "gemm"): 4.486e8,     # FETCH 217,244.9 x 2.000 KiB + WRITE 3,627.6 x 1.000 KiB
-    ("c4", "gemm"): 1.458e9,     # FETCH 678,663.1 x 2.000 KiB + WRITE 66,279.4 x 1.000 KiB
-    ("c4", "quant"): 1.786e8,    # FETCH 57,400.1 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
+    ("c1", "gemm"): 1.563e9,     # FETCH 736,665.2 x 2.000 KiB + WRITE 53,224.2 x 1.000 KiB
+    ("c2", "gemm"): 4.487e8,     # FETCH 217,295.2 x 2.000 KiB + WRITE 3,627.5 x 1.000 KiB
+    ("c4", "gemm"): 1.457e9,     # FETCH 678,291.3 x 2.000 KiB + WRITE 66,255.0 x 1.000 KiB
+    ("c4", "quant"): 1.786e8,    # FETCH 57,399.0 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
 }
+
+
+def settle(step, ms):
+    """Untimed: keeps the GPU on this step's work for `ms` milliseconds before the warm-up steps.  A chip that has
+    been idle runs its first tens of milliseconds of work at lower clocks, whatever the number of warm-up steps."""
+    if ms <= 0:
+        return
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
 
 
 def calibration_copy():
@@ -38,8 +50,13 @@ def calibration_copy():
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=300,
+                    help="untimed steps before the timed ones; the chip needs some tens of milliseconds of this work before its "
+                         "clocks settle (C1: 314 us per step after 5 warm-up steps, 285 after 50, 276 after 500)")
+    ap.add_argument("--settle-ms", type=float, default=200.0,
+                    help="untimed: run the step for this many milliseconds before the warm-up steps, so that a small "
+                         "--warmup does not time the chip's clock ramp (0 = off)")
     ap.add_argument("--config", default="c1", choices=["c1", "c2", "c3", "c4"])
     ap.add_argument("--tokens", type=int, default=8192, help="c3 only")
     ap.add_argument("--routing", default="zipf", choices=["zipf", "uniform"], help="c3 only")
@@ -143,6 +160,7 @@ def bench_quant(args, prob, es, W):
         else:
             es.es_sm100_mxfp8_blockscaled_grouped_quant(xd, ps, eo, bso, q, sf)
 
+    settle(step, args.settle_ms)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -164,7 +182,7 @@ def bench_quant(args, prob, es, W):
     out = {
         "metric": ("FP8 1x128 activation quantisation, algorithmic GB/s (bf16 in, e4m3 + fp32 scales out)" if act else
                    "MXFP8 grouped quantisation, algorithmic GB/s (bf16 in, e4m3 + E8M0 out)"),
-        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_ms": args.settle_ms,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 -> fp8_e4m3 + fp32 scales" if act else "bf16 -> fp8_e4m3 + e8m0", "data": "synthetic",
         "config": {"workload": f"{prob.name} {args.op}: E={len(rows)} K={k} rows={total} max_rows={max(rows)} seed={args.seed}"},
@@ -212,6 +230,7 @@ def bench_swiglu_quant(args, prob, es, W):
         else:
             es.es_swiglu_quant_1x128(xd, q, sc)
 
+    settle(step, args.settle_ms)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -233,7 +252,7 @@ def bench_swiglu_quant(args, prob, es, W):
     out = {
         "metric": ("fused SwiGLU + MXFP8 grouped quantisation, algorithmic GB/s (bf16 [rows, 2I] in, e4m3 + E8M0 scales out)" if mx else
                    "fused SwiGLU + FP8 1x128 quantisation, algorithmic GB/s (bf16 [rows, 2I] in, e4m3 + fp32 scales out)"),
-        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_ms": args.settle_ms,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 -> fp32 -> bf16 -> fp8_e4m3 + " + ("e8m0 scales" if mx else "fp32 scales"), "data": "synthetic",
         "config": {"workload": f"{prob.name} swiglu_quant: rows={total} inter={inter} seed={args.seed}"},
@@ -278,6 +297,7 @@ def bench_route(args, prob, es, W):
         ps, eo, bso, dst = es.es_route_metadata(d_ids, 0, e, n, k)
         es.es_permute_rows(x, dst, 1, packed)
 
+    settle(step, args.settle_ms)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -298,7 +318,7 @@ def bench_route(args, prob, es, W):
     roof["roofline_us"] = nbytes / W.HBM_BYTES_PER_S * 1e6
     out = {
         "metric": "routing metadata + row packing, algorithmic GB/s (4 kernels)",
-        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_ms": args.settle_ms,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int32 ids, bf16 rows", "data": "synthetic",
         "config": {"workload": f"{prob.name} route: E={e} K={k} pairs={total} seed={args.seed}"},
@@ -339,6 +359,7 @@ def bench_quant_weight(args, prob, es, W):
         else:
             es.es_fp8_quant_weight_128x128(w, q, sc)
 
+    settle(step, args.settle_ms)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -360,7 +381,7 @@ def bench_quant_weight(args, prob, es, W):
     out = {
         "metric": ("MXFP8 weight quantisation, algorithmic GB/s (bf16 in, e4m3 + E8M0 scales out)" if mx else
                    "FP8 128x128 weight quantisation, algorithmic GB/s (bf16 in, e4m3 + fp32 scales out)"),
-        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": nbytes / t / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_ms": args.settle_ms,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 -> fp8_e4m3 + " + ("e8m0 scales" if mx else "fp32 scales"), "data": "synthetic",
         "config": {"workload": f"{prob.name} quant_weight: E={e} N={n} K={k} seed={args.seed}"},
@@ -485,6 +506,7 @@ def main():
                                                   ops["stride_a"], ops["stride_b"], ops["stride_d"],
                                                   ops["problem_sizes"], ops["expert_offsets"], ops["workspace"])
 
+    settle(step, args.settle_ms)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -519,7 +541,7 @@ def main():
     roof["per_expert_roofline_us"] = W.gemm_roofline_per_expert_seconds(prob.rows, n, k, prob.kind) * 1e6
     out = {
         "metric": "useful FP8 TFLOP/s + % of roofline, DSv3-shape grouped GEMM, Zipf routing",
-        "value": flops / t / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": flops / t / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_ms": args.settle_ms,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8_e4m3 (fp32 accumulate, bf16 out)", "data": "synthetic",
         "config": {"workload": f"{prob.name}: E={e} K={k} N={n} rows={total} max_rows={max(prob.rows)} "
