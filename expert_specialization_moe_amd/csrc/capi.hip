@@ -80,7 +80,7 @@ int current_device_info(DeviceInfo* out) {
 // ESMOE_* environment variables (tuning aids) are read once per process, on the first GEMM launch; a value the
 // kernels cannot honour is reported by every launch instead of being applied.
 struct Knobs {
-  int big_mt_fp8 = 12, big_mt_mx = 12, order = 0, light_share = -1, wgs_per_cu = 1;
+  int big_mt_fp8 = 12, big_mt_mx = 12, order = 0, light_share = -1, wgs_per_cu = 1, narrow_tail = -1;
   char error[160] = "";
 };
 
@@ -101,6 +101,8 @@ const Knobs& knobs() {
     if (r.order < 0 || r.order > 2) snprintf(r.error, sizeof(r.error), "ESMOE_ORDER must be 0, 1 or 2");
     r.light_share = env_int("ESMOE_LIGHT_SHARE", -1);
     if (r.light_share < -1 || r.light_share > 32) snprintf(r.error, sizeof(r.error), "ESMOE_LIGHT_SHARE must be in [-1, 32]");
+    r.narrow_tail = env_int("ESMOE_NARROW_TAIL", -1);
+    if (r.narrow_tail < -1 || r.narrow_tail > 65536) snprintf(r.error, sizeof(r.error), "ESMOE_NARROW_TAIL must be in [-1, 65536]");
     r.wgs_per_cu = env_int("ESMOE_WGS_PER_CU", 1);
     if (r.wgs_per_cu < 1 || r.wgs_per_cu > 8) snprintf(r.error, sizeof(r.error), "ESMOE_WGS_PER_CU must be in [1, 8]");
     return r;
@@ -108,8 +110,12 @@ const Knobs& knobs() {
   return k;
 }
 
-// Default schedule policy: the one the host mirrors describe.
-esmoe::SchedPolicy default_policy(int force_bm, int mx) {
+// Light items of a launch's tail that go out as two 128-column halves (schedule.h); about half a launch's workgroups.
+constexpr int kNarrowTail = 128;
+
+// Default schedule policy: the one the host mirrors describe.  kind: bit 0 mxfp8, bit 1 a fused SwiGLU epilogue.
+esmoe::SchedPolicy default_policy(int force_bm, int kind) {
+  const int mx = kind & 1;
   esmoe::SchedPolicy p;
   p.force_mt = force_bm / 16;
   // Full tiles are 192 rows for both kernels: the tallest tile whose ring (three weight stages, two token stages per
@@ -119,14 +125,17 @@ esmoe::SchedPolicy default_policy(int force_bm, int mx) {
   p.big_mt = 12;
   p.order = 0;
   p.light_share = -1;
+  // the fused epilogues quantise blocks that need a whole 256-row tile, and a forced height has no light items
+  p.narrow_tail = (force_bm == 0 && !(kind & 2)) ? kNarrowTail : 0;
   return p;
 }
 
 // Policy of a launch: the default with the environment's overrides.
-esmoe::SchedPolicy launch_policy(int force_bm, int mx) {
-  esmoe::SchedPolicy p = default_policy(force_bm, mx);
+esmoe::SchedPolicy launch_policy(int force_bm, int kind) {
+  esmoe::SchedPolicy p = default_policy(force_bm, kind);
   const Knobs& k = knobs();
-  p.big_mt = mx ? k.big_mt_mx : k.big_mt_fp8;
+  p.big_mt = (kind & 1) ? k.big_mt_mx : k.big_mt_fp8;
+  if (p.narrow_tail && k.narrow_tail >= 0) p.narrow_tail = k.narrow_tail;
   p.order = k.order;
   p.light_share = k.light_share;
   return p;
@@ -160,7 +169,7 @@ int launch_gemm(esmoe::GemmArgs& g, int mx, int force_bm, void* stream) {
   int rc = current_device_info(&info);
   if (rc) return rc;
   if (knobs().error[0]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "%s", knobs().error);
-  g.policy = launch_policy(force_bm, mx);
+  g.policy = launch_policy(force_bm, (mx ? 1 : 0) | (g.q_out ? 2 : 0));
   int grid = info.cus * knobs().wgs_per_cu;
   rc = esmoe_launch_grouped_gemm(&g, mx, grid, (hipStream_t)stream);
   if (rc) return fail(rc, "grouped GEMM launch failed: %s", hipGetErrorString((hipError_t)rc));
@@ -448,12 +457,12 @@ int esmoe_permute_rows(const void* in, const int32_t* dst_row, long num_pairs, i
   return 0;
 }
 
-int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int mx,
+int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int kind,
                         int32_t* ws_host) {
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS || n <= 0 || n % 128)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_schedule");
-  const esmoe::SchedPolicy p = default_policy(force_bm, mx != 0);
+  const esmoe::SchedPolicy p = default_policy(force_bm, kind);
   auto rows_of = [&](int e) { return problem_sizes_host[e * 3] < 0 ? 0 : problem_sizes_host[e * 3]; };
   // same ranking as the device schedule kernel: by sched_order_key, ties by expert index
   for (int e = 0; e < num_experts; e++) {
@@ -487,7 +496,9 @@ int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int 
   last[esmoe::kRecRows] = 0;
   ws_host[esmoe::kWsLightShare] = esmoe::sched_light_share(heavy_cost, light_cost, p);
   ws_host[esmoe::kWsHeavyBlocks] = blocks;
-  ws_host[esmoe::kWsLightTotal] = items;
+  const int split = esmoe::sched_light_split(items, p);
+  ws_host[esmoe::kWsLightSplit] = split;
+  ws_host[esmoe::kWsLightTotal] = split + 2 * (items - split);
   ws_host[esmoe::kWsLightCounter] = 0;
   for (int x = 0; x < esmoe::kXcds; x++) ws_host[esmoe::kWsXcdCounter + x] = 0;
   return 0;
@@ -506,11 +517,11 @@ void fill_out5(int32_t* out5, int e, const esmoe::TileCoord& t) {
 }  // namespace
 
 int esmoe_host_decode_heavy(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                            int force_bm, int mx, int xcd, int ticket, int32_t* out5) {
+                            int force_bm, int kind, int xcd, int ticket, int32_t* out5) {
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || !out5 || xcd < 0 || xcd >= esmoe::kXcds || ticket < 0)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "bad argument to esmoe_host_decode_heavy");
-  const esmoe::SchedPolicy p = default_policy(force_bm, mx != 0);
+  const esmoe::SchedPolicy p = default_policy(force_bm, kind);
   const int blk = esmoe::sched_ticket_block(xcd, ticket);
   if (blk >= ws_host[esmoe::kWsHeavyBlocks]) return 2;   // this XCD's queue is exhausted
   const int pos = host_position(ws_host, num_experts, esmoe::kRecBlock, blk);
@@ -524,16 +535,19 @@ int esmoe_host_decode_heavy(const int32_t* problem_sizes_host, const int32_t* ws
 }
 
 int esmoe_host_decode_light(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                            int force_bm, int mx, int item, int32_t* out5) {
+                            int force_bm, int kind, int item, int32_t* out5) {
   g_err[0] = 0;
   if (!problem_sizes_host || !ws_host || !out5) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null pointer");
-  (void)n;
-  const esmoe::SchedPolicy p = default_policy(force_bm, mx != 0);
+  const esmoe::SchedPolicy p = default_policy(force_bm, kind);
   if (item < 0 || item >= ws_host[esmoe::kWsLightTotal]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "item out of range");
-  const int pos = host_position(ws_host, num_experts, esmoe::kRecItem, item);
+  int half = -1;
+  const int idx = esmoe::sched_light_item_of_ticket(item, ws_host[esmoe::kWsLightSplit], &half);
+  const int pos = host_position(ws_host, num_experts, esmoe::kRecItem, idx);
   if (pos < 0) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace does not hold a schedule");
   const int32_t* rec = ws_host + esmoe::ws_rec(pos);
-  fill_out5(out5, rec[esmoe::kRecExpert], esmoe::sched_decode_light(item - rec[esmoe::kRecItem], rec[esmoe::kRecRows], p));
+  const esmoe::TileCoord t = esmoe::sched_decode_light(idx - rec[esmoe::kRecItem], rec[esmoe::kRecRows], p, half);
+  if (t.n0 >= n) return 1;   // second half of a last column tile that is 128 columns wide: skipped
+  fill_out5(out5, rec[esmoe::kRecExpert], t);
   return 0;
 }
 

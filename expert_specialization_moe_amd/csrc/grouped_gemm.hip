@@ -142,23 +142,27 @@ __device__ __forceinline__ void block_barrier() {
 
 // Shape of a short tile (MT*16 <= 64 token rows) and the layout of one ring stage (token rows, weight rows, scales):
 // each of the 8 wavefronts has all token rows and 32 weight rows.  (Tall tiles: gemm_tile_pp, gemm_tile_pp_mx.)
-template <int MT, bool MX>
+template <int MT, bool MX, int BN = kBN>
 struct TileGeom {
+  static_assert(BN == 256 || BN == 128, "tile widths: 256 weight rows, or 128 for the narrow items that end a launch");
   static constexpr int BM = MT * 16;
   static constexpr int kWavesM = 1;
   static constexpr int kWavesN = kWaves / kWavesM;
   static constexpr int MTW = MT / kWavesM;          // row tiles per wavefront
-  static constexpr int NTW = kBN / 16 / kWavesN;    // weight-row tiles per wavefront
+  static constexpr int NTW = BN / 16 / kWavesN;     // weight-row tiles per wavefront
   static constexpr int kABytes = BM * 128;
-  static constexpr int kWBytes = kBN * 128;
+  static constexpr int kWBytes = BN * 128;
   // scales of one K block: fp8-blockwise -> 256 floats (sa of the tile's rows); mxfp8 -> verbatim
   // 512-byte swizzled scale tiles, 2 for the weight rows then up to 2 for the token rows
   static constexpr int kScaleBytes = MX ? 2048 : 1024;
   static constexpr int kStageBytes = kABytes + kWBytes + kScaleBytes;
-  static constexpr int kNBuf = ring_bytes<MX>() / kStageBytes >= 4 ? 4 : ring_bytes<MX>() / kStageBytes;
+  // (a fifth stage for the narrow tile, whose stages are half the bytes; more would let a scale chunk, fetched four K
+  // blocks ahead, be younger than the stages the loop's waits leave in flight)
+  static constexpr int kMaxBuf = BN == 128 ? 5 : 4;
+  static constexpr int kNBuf = ring_bytes<MX>() / kStageBytes >= kMaxBuf ? kMaxBuf : ring_bytes<MX>() / kStageBytes;
   static constexpr int kABlocks = BM / 8;                               // 8-row copy blocks of the token tile
   static constexpr int kACopies = kABlocks >= kWaves ? kABlocks / kWaves : 1;  // per wavefront
-  static constexpr int kWCopies = kBN / 8 / kWaves;                     // 4
+  static constexpr int kWCopies = BN / 8 / kWaves;                      // 4 (2 for the narrow tile)
   static constexpr int kCopiesPerStage = kACopies + kWCopies + 1;       // + 1 scale copy
   static_assert(kNBuf >= 2, "ring too small");
 };
@@ -343,10 +347,11 @@ __device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, i
 // rows and the matching 128 up rows, interleaved so that every wavefront holds gate and up of the same columns; the
 // epilogue forms silu(gate) * up and quantises it for the down projection (fp8-blockwise: 1x128 blocks with fp32
 // scales, tile_epilogue; mxfp8: 1x32 blocks with E8M0 scales, tile_epilogue_mxq) instead of writing the projection.
-template <int MT, bool MX, bool FUSE>
+template <int MT, bool MX, bool FUSE, int BN = kBN>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds) {
+  static_assert(!(FUSE && BN != kBN), "the fused epilogues need gate and up columns of a whole quantisation block in one tile");
   static_assert(MT == 1 || MT == 2 || MT == 4, "short tiles; 128- and 192-row tiles are gemm_tile_pp / gemm_tile_pp_mx");
-  using G = TileGeom<MT, MX>;
+  using G = TileGeom<MT, MX, BN>;
   constexpr int MTW = G::MTW, NTW = G::NTW, NBUF = G::kNBuf;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -449,7 +454,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   const bool w_once = m0 == 0 && M <= G::BM;   // the expert is one tile high: nobody else reads these weight rows
   auto issue_w = [&](int kb, int buf) {
     const uint32_t lw = lds0 + buf * G::kStageBytes + G::kABytes + wave * G::kWCopies * 1024;
-    static_assert(G::kWCopies == 4, "weight copies per wavefront");
     if (w_once) dma16xn<true>(lw, w_ptr + (long)kb * 128, vw);
     else dma16xn<false>(lw, w_ptr + (long)kb * 128, vw);
   };
@@ -1112,7 +1116,9 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
       ws[ws_rec(num_experts) + kRecExpert] = -1;
       ws[ws_rec(num_experts) + kRecRows] = 0;
       ws[kWsHeavyBlocks] = blocks;
-      ws[kWsLightTotal] = items;
+      const int split = sched_light_split(items, policy);
+      ws[kWsLightSplit] = split;
+      ws[kWsLightTotal] = split + 2 * (items - split);
       ws[kWsLightCounter] = 0;
       long heavy_cost = 0, light_cost = 0;
       for (int j = 0; j < num_experts; j++) {
@@ -1146,7 +1152,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   __shared__ int s_counters[kXcds + 1];
   int* ws = g.ws;
   const int hblocks = ws[kWsHeavyBlocks];
-  const int ltotal = ws[kWsLightTotal];
+  const int ltotal = ws[kWsLightTotal], lsplit = ws[kWsLightSplit];
 #define ESMOE_CASE(MT_) \
   case (MT_): gemm_tile<MT_, MX, FUSE>(g, e, M, t.m0, t.n0, lds); break;
 
@@ -1211,18 +1217,30 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     // schedule position of v: the last one whose first block (item) is <= v, found by bisection over the prefix
     // sums with scalar loads.  The records are written by the schedule kernel and only read here, so they stay in
     // the scalar cache, where a step costs a fraction of what a trip to L2 costs while the chip streams weights.
+    // (a light ticket past `lsplit` is one half of an item of the narrow tail)
+    int half = -1;
+    const int idx = light ? sched_light_item_of_ticket(v, lsplit, &half) : v;
     int lo = 0, hi = g.num_experts;
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
-      if (sload(ws, (ws_rec(mid) + kind) * 4) <= v) lo = mid; else hi = mid;
+      if (sload(ws, (ws_rec(mid) + kind) * 4) <= idx) lo = mid; else hi = mid;
     }
     const int first = sload(ws, (ws_rec(lo) + kind) * 4);
     const int e = sload(ws, (ws_rec(lo) + kRecExpert) * 4), M = sload(ws, (ws_rec(lo) + kRecRows) * 4);
-    const int local = v - first;
+    const int local = idx - first;
     TileCoord t;
-    if (light) t = sched_decode_light(local, M, g.policy);
+    if (light) t = sched_decode_light(local, M, g.policy, half);
     else if (!sched_decode_heavy(local, ticket % kBlkTiles, M, g.n, g.policy, &t)) {
       __syncthreads();   // s_item is rewritten next: every wavefront must have read this ticket first
+      continue;
+    }
+    // (wave-uniform by construction; said again so that the copies' base pointers stay in scalar registers)
+    t.mt = __builtin_amdgcn_readfirstlane(t.mt);
+    t.nt = __builtin_amdgcn_readfirstlane(t.nt);
+    t.m0 = __builtin_amdgcn_readfirstlane(t.m0);
+    t.n0 = __builtin_amdgcn_readfirstlane(t.n0);
+    if (t.n0 >= g.n) {   // second half of a last column tile that is 128 columns wide
+      __syncthreads();
       continue;
     }
 #ifdef ESMOE_TIMELINE
@@ -1252,9 +1270,20 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
       }
     }
     if (!hand_scheduled) {
-      switch (t.mt) {
-        ESMOE_VARIANTS
-        default: break;
+      if (!FUSE && t.nt == 2) {
+        if constexpr (!FUSE) {
+          switch (t.mt) {
+            case 1: gemm_tile<1, MX, false, 128>(g, e, M, t.m0, t.n0, lds); break;
+            case 2: gemm_tile<2, MX, false, 128>(g, e, M, t.m0, t.n0, lds); break;
+            case 4: gemm_tile<4, MX, false, 128>(g, e, M, t.m0, t.n0, lds); break;
+            default: break;
+          }
+        }
+      } else {
+        switch (t.mt) {
+          ESMOE_VARIANTS
+          default: break;
+        }
       }
     }
 #ifdef ESMOE_TIMELINE

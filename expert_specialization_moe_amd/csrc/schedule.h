@@ -29,6 +29,7 @@ struct SchedPolicy {
   int order;      // 0: heavy experts by rows ascending, light ones descending (sched_order_key); 1: expert index order;
                   // 2: most rows first for both kinds
   int light_share;  // workgroups (of every 32) that start on the light items; -1 = from the cost estimate
+  int narrow_tail;  // the last so many light items are handed out as two 128-column halves each (0: none)
 };
 
 struct TileCoord {
@@ -133,12 +134,31 @@ ESMOE_HD bool sched_decode_heavy(int lb, int idx, int m, int n, const SchedPolic
   return true;
 }
 
-ESMOE_HD TileCoord sched_decode_light(int item, int m, const SchedPolicy& p) {
+// Light items are handed out whole (256 columns) except the last `narrow_tail` of the launch, which go out as two
+// 128-column halves each: a launch ends on light items (they are the last of the light-first workgroups' queue, and
+// what the others turn to when the heavy tickets are gone), fewer of them are left than there are workgroups, and an
+// item holds a CU for as long as a tall tile, so halves spread the end of the launch over twice the CUs.
+// Tickets [0, split) are the whole items 0 .. split-1, tickets split + 2j and split + 2j + 1 the halves of item split + j.
+ESMOE_HD int sched_light_split(int items, const SchedPolicy& p) {
+  const int narrow = p.narrow_tail < items ? p.narrow_tail : items;
+  return items - (narrow > 0 ? narrow : 0);
+}
+ESMOE_HD int sched_light_item_of_ticket(int ticket, int split, int* half) {
+  if (ticket < split) {
+    *half = -1;
+    return ticket;
+  }
+  *half = (ticket - split) & 1;
+  return split + ((ticket - split) >> 1);
+}
+
+// Item `item` of a light expert; half = -1: the whole 256-column item, 0 / 1: its first / second 128 columns.
+ESMOE_HD TileCoord sched_decode_light(int item, int m, const SchedPolicy& p, int half = -1) {
   TileCoord t;
   t.mt = sched_cover_mt(m, p.big_mt);
-  t.nt = 4;
+  t.nt = half < 0 ? 4 : 2;
   t.m0 = 0;
-  t.n0 = item * 256;
+  t.n0 = item * 256 + (half > 0 ? 128 : 0);
   return t;
 }
 
@@ -168,9 +188,10 @@ ESMOE_HD int sched_ticket_block(int xcd, int ticket) { return (ticket / kBlkTile
 
 // Workspace layout (int32 words).
 constexpr int kWsLightCounter = 0;   // next light item to hand out
-constexpr int kWsLightTotal = 1;     // number of light items
+constexpr int kWsLightTotal = 1;     // number of light tickets: whole items, then two per item of the narrow tail
 constexpr int kWsHeavyBlocks = 2;    // number of heavy blocks
 constexpr int kWsLightShare = 3;     // workgroups of every 32 that start on the light items
+constexpr int kWsLightSplit = 4;     // first light ticket that is a half item (sched_light_split)
 constexpr int kWsXcdCounter = 8;     // 8 words: next heavy ticket of every XCD
 constexpr int kWsHeader = 16;        // then one record of kRecWords per schedule position, E + 1 of them
 // Record of schedule position p: first heavy block, first light item, expert index, rows (clamped at 0).

@@ -250,18 +250,22 @@ int esmoe_permute_rows(const void* in, const int32_t* dst_row, long num_pairs, i
  * to XCD b % 8, through one ticket counter per XCD; esmoe_host_decode_heavy maps ticket `ticket` of XCD `xcd`
  * to out5 = {expert, tile rows, tile cols, m0, n0} and returns 0, or 1 if the ticket falls outside the
  * expert's tile grid (the kernel skips it), or 2 if that XCD's queue is exhausted.
- * The other experts are "light": one short tile per 256 columns from a launch-wide counter;
- * esmoe_host_decode_light maps item `item` (< word 1 of the workspace) to out5.
- * mx: 0 describes the FP8-blockwise launch, 1 the MXFP8 launch (both cut experts into full tiles of 192 rows today).
+ * The other experts are "light": one short tile per 256 columns from a launch-wide counter, except that the last 128
+ * light items of a launch go out as two 128-column halves each (word 4 of the workspace is the first ticket that is a
+ * half, word 1 the number of light tickets); esmoe_host_decode_light maps ticket `item` (< word 1) to out5 and returns
+ * 0, or 1 for the second half of a last column tile that is only 128 columns wide (the kernel skips it).
+ * kind: bit 0 clear describes the FP8-blockwise launch, set the MXFP8 launch (both cut experts into full tiles of 192
+ * rows today); bit 1 set describes a launch with a fused SwiGLU epilogue, whose items all stay 256 columns wide, as do
+ * those of a launch with a forced tile height.
  * The mirrors describe the default policy; the ESMOE_* environment variables, which a launch reads once per process, do not
  * reach them.
  */
-int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int mx,
+int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int n, int force_bm, int kind,
                         int32_t* ws_host);
 int esmoe_host_decode_heavy(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                            int force_bm, int mx, int xcd, int ticket, int32_t* out5);
+                            int force_bm, int kind, int xcd, int ticket, int32_t* out5);
 int esmoe_host_decode_light(const int32_t* problem_sizes_host, const int32_t* ws_host, int num_experts, int n,
-                            int force_bm, int mx, int item, int32_t* out5);
+                            int force_bm, int kind, int item, int32_t* out5);
 
 /* Message describing the calling thread's most recent failure ("" if none). */
 const char* esmoe_last_error(void);
