@@ -3,7 +3,7 @@
 // One launch serves every expert.  A one-workgroup schedule kernel turns problem_sizes into a list of workgroup
 // tiles (schedule.h); persistent workgroups of 8 wavefronts then pull tiles from atomic counters.  A tile is
 // (MT*16) token rows x 256 weight rows, MT in {1, 2, 4} (short tiles, gemm_tile) or {8, 12} (tall tiles,
-// gemm_tile_pp / gemm_tile_pp_mx).
+// gemm_tile_pp / gemm_tile_pp_mx); the short items that end a launch are handed out as two 128-column halves.
 //
 // Data movement.  Per 128-wide K block the workgroup copies the token rows, the weight rows and the block's scales
 // of its tile from global memory straight into LDS with global_load_lds (no staging registers, no LDS store
