@@ -283,3 +283,28 @@ def test_graph_capture_replays_match_eager(esmoe, kind):
         assert np.isfinite(scratch)
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {rep} differs from the eager result"
+
+
+@pytest.mark.parametrize("kind", ["fp8", "mx"])
+@pytest.mark.parametrize("n", [1024, 1152])
+def test_half_items_give_the_bytes_of_whole_items(esmoe, kind, n):
+    """A plain launch hands its last 128 light items out as 128-column halves; a launch with a forced tile height hands out
+    whole tiles only.  On experts of at most 16 rows both use 16-row tiles with the same K order, so the outputs must be
+    identical bit for bit.  44 experts x 4-5 column tiles: whole items, then halves; n = 1152 ends on a 128-column tile
+    whose second half is skipped."""
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import workloads as W
+
+    rows = [1 + (7 * i) % 16 for i in range(44)]
+    rows[5] = 0
+    prob = W.Problem("halves", n, 768, rows, kind="mxfp8" if kind == "mx" else "fp8_blockwise")
+    if kind == "mx":
+        ops = W.make_mxfp8_operands(prob, "cuda", seed=21, weight_std=0.05)
+        mm = H.capi_mx_mm
+    else:
+        ops = W.make_fp8_blockwise_operands(prob, "cuda", seed=21, weight_std=0.05)
+        mm = H.capi_fp8_mm
+    y0 = mm(_native, ops, 0, out=torch.full_like(ops["output"], 7.0)).clone()
+    y16 = mm(_native, ops, 16, out=torch.full_like(ops["output"], 7.0)).clone()
+    assert torch.equal(y0.view(torch.int16), y16.view(torch.int16))
+    assert not (y0 == 7.0).all(dim=1).any()      # every row of an expert was written
