@@ -500,7 +500,7 @@ int esmoe_host_schedule(const int32_t* problem_sizes_host, int num_experts, int 
   ws_host[esmoe::kWsLightSplit] = split;
   ws_host[esmoe::kWsLightTotal] = split + 2 * (items - split);
   ws_host[esmoe::kWsLightCounter] = 0;
-  for (int x = 0; x < esmoe::kXcds; x++) ws_host[esmoe::kWsXcdCounter + x] = 0;
+  for (int x = 0; x < esmoe::kXcds; x++) ws_host[esmoe::ws_xcd_counter(x)] = 0;
   return 0;
 }
 

@@ -1127,9 +1127,9 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
       }
       ws[kWsLightShare] = sched_light_share(heavy_cost, light_cost, policy);
     }
-    if (pos < kXcds) ws[kWsXcdCounter + pos] = 0;
+    if (pos < kXcds) ws[ws_xcd_counter(pos)] = 0;
   }
-  if (num_experts < kXcds && e >= num_experts && e < kXcds) ws[kWsXcdCounter + e] = 0;
+  if (num_experts < kXcds && e >= num_experts && e < kXcds) ws[ws_xcd_counter(e)] = 0;
 }
 
 // Heights whose fp8-blockwise tiles run the hand-scheduled K block of gemm_tile_pp (bit 0: 128 rows, bit 1: 192 rows).
@@ -1185,7 +1185,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
       }
       continue;
     }
-    if (threadIdx.x == 0) s_item = atomicAdd(light ? &ws[kWsLightCounter] : &ws[kWsXcdCounter + xq], 1);
+    if (threadIdx.x == 0) s_item = atomicAdd(light ? &ws[kWsLightCounter] : &ws[ws_xcd_counter(xq)], 1);
     __syncthreads();
     const int ticket = __builtin_amdgcn_readfirstlane(s_item);
     const int kind = light ? kRecItem : kRecBlock;
@@ -1202,7 +1202,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
       // (worth its round trip only when every XCD has a queue to try: the look itself reads the hot counter line)
       if (hblocks <= kXcds) continue;
       if (threadIdx.x < kXcds + 1)
-        s_counters[threadIdx.x] = __hip_atomic_load(threadIdx.x < kXcds ? &ws[kWsXcdCounter + threadIdx.x] : &ws[kWsLightCounter],
+        s_counters[threadIdx.x] = __hip_atomic_load(threadIdx.x < kXcds ? &ws[ws_xcd_counter(threadIdx.x)] : &ws[kWsLightCounter],
                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
 #pragma unroll

@@ -187,17 +187,18 @@ ESMOE_HD int sched_light_share(long heavy_cost, long light_cost, const SchedPoli
 ESMOE_HD int sched_ticket_block(int xcd, int ticket) { return (ticket / kBlkTiles) * kXcds + xcd; }
 
 // Workspace layout (int32 words).
-constexpr int kWsLightCounter = 0;   // next light item to hand out
+constexpr int kWsLightCounter = 32;  // next light ticket to hand out (every counter has a 128-byte line of its own)
 constexpr int kWsLightTotal = 1;     // number of light tickets: whole items, then two per item of the narrow tail
 constexpr int kWsHeavyBlocks = 2;    // number of heavy blocks
 constexpr int kWsLightShare = 3;     // workgroups of every 32 that start on the light items
 constexpr int kWsLightSplit = 4;     // first light ticket that is a half item (sched_light_split)
-constexpr int kWsXcdCounter = 8;     // 8 words: next heavy ticket of every XCD
-constexpr int kWsHeader = 16;        // then one record of kRecWords per schedule position, E + 1 of them
+constexpr int kWsXcdCounter = 64;    // next heavy ticket of XCD x at word kWsXcdCounter + 32 * x (ws_xcd_counter)
+constexpr int kWsHeader = 64 + 32 * kXcds;   // then one record of kRecWords per schedule position, E + 1 of them
 // Record of schedule position p: first heavy block, first light item, expert index, rows (clamped at 0).
 // Record E closes the prefix sums: {heavy blocks, light items, -1, 0}.
 constexpr int kRecWords = 4;
 constexpr int kRecBlock = 0, kRecItem = 1, kRecExpert = 2, kRecRows = 3;
+ESMOE_HD int ws_xcd_counter(int xcd) { return kWsXcdCounter + 32 * xcd; }
 ESMOE_HD int ws_rec(int pos) { return kWsHeader + pos * kRecWords; }
 ESMOE_HD int ws_words(int num_experts) { return kWsHeader + (num_experts + 1) * kRecWords; }
 
