@@ -484,12 +484,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // The work on one K block is split in two phases, so that the two groups of four wavefronts (one
   // wavefront of each group per SIMD) can run half an iteration apart: while one group's MFMAs keep
   // the matrix pipe busy, the other group reads its fragments from LDS.
-  //   read phase: weight fragments, the first kPre token fragments and all scales -> registers
+  //   read phase: weight fragments, token fragments and all scales -> registers (every fragment of a short tile fits)
   //   mfma phase: the MFMAs (+ the fp32 promotion for fp8-blockwise) of the K block
-  constexpr int kPre = MTW;   // every token fragment of a short tile fits in registers
   struct Frags {
     v8i wf[NTW];
-    v8i af[kPre];
+    v8i af[MTW];
     int sfw[MX ? NTW : 1];
     int sfa[MX ? MTW : 1];
     float sc[MX ? 1 : MTW];   // fp8-blockwise: sa of the row tiles (the product with sb is formed in the mfma phase)
@@ -515,7 +514,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       f.wf[nt] = join(*(const v4i*)(lb + wfrag_lo + nt * 2048), *(const v4i*)(lb + (wfrag_lo ^ 64) + nt * 2048));
     }
 #pragma unroll
-    for (int mt = 0; mt < kPre; mt++) {
+    for (int mt = 0; mt < MTW; mt++) {
       f.af[mt] = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + (afrag_lo ^ 64) + mt * 2048));
     }
     if constexpr (MX) {
@@ -539,14 +538,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     }
   };
 
-  // fp8-blockwise with all fragments in registers: MFMAs and promotions form one scheduling region in which
-  // the four v_fmac of MFMA j - 3 follow MFMA j, so the vector ALU works in the shadow of the matrix pipe
-  // and no promotion waits on the MFMA it has just been issued behind.  Taller tiles (fragments read from
-  // LDS during the phase) keep the coarser order: promotion of row tile mt behind the MFMAs of mt + 1.
-  auto mfma_phase = [&](int buf, const Frags& f) {
-    const uint8_t* lb = lds + buf * G::kStageBytes;
-    if constexpr (!MX && kPre == MTW) {
-      // all fragments are in registers: one scheduling region in which promotion j - LAG issues behind MFMA j
+  // fp8-blockwise: MFMAs and promotions form one scheduling region in which the four v_fmac of MFMA j - 3 follow
+  // MFMA j, so the vector ALU works in the shadow of the matrix pipe and no promotion waits on the MFMA it has just been
+  // issued behind.  mxfp8: the scaled MFMA accumulates in place.
+  auto mfma_phase = [&](const Frags& f) {
+    if constexpr (!MX) {
       float sc[MTW], sc_up[FUSE ? MTW : 1];
 #pragma unroll
       for (int mt = 0; mt < MTW; mt++) {
@@ -566,7 +562,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
           for (int i = 0; i < 4; i++)
             acc[nt][mt][i] = __builtin_fmaf(t[mt][nt][i], (FUSE && nt >= NTW / 2) ? sc_up[FUSE ? mt : 0] : sc[mt], acc[nt][mt][i]);
-      constexpr int kT = MTW * NTW, kLag = 3;
+      constexpr int kT = MTW * NTW, kLag = kT < 3 ? kT : 3;
 #pragma unroll
       for (int j = 0; j < kLag; j++) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 #pragma unroll
@@ -580,46 +576,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       for (int mt = 0; mt < MTW; mt++)
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++) asm volatile("" : "+v"(acc[nt][mt]));   // the promotions stay in this phase
-      return;
-    }
-    v4f tmp[2][NTW];
+    } else {
 #pragma unroll
-    for (int mt = 0; mt < MTW; mt++) {
-      v8i afr;
-      if (mt < kPre) afr = f.af[mt < kPre ? mt : 0];
-      else afr = join(*(const v4i*)(lb + afrag_lo + mt * 2048), *(const v4i*)(lb + (afrag_lo ^ 64) + mt * 2048));
-      if constexpr (!MX) {
+      for (int mt = 0; mt < MTW; mt++) {
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++) {
-          tmp[mt & 1][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], afr, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], f.af[mt], acc[nt][mt], 0, 0, 0, f.sfw[nt], 0, f.sfa[mt]);
         }
-      } else {
-#pragma unroll
-        for (int nt = 0; nt < NTW; nt++) {
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f.wf[nt], afr, acc[nt][mt], 0, 0, 0, f.sfw[nt], 0, f.sfa[mt]);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (!MX) {
-        if (mt > 0) {
-#pragma unroll
-          for (int nt = 0; nt < NTW; nt++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-              acc[nt][mt - 1][i] = __builtin_fmaf(tmp[(mt - 1) & 1][nt][i], f.sc[mt - 1] * ((FUSE && nt >= NTW / 2) ? f.sb_up : f.sb), acc[nt][mt - 1][i]);
-            asm volatile("" : "+v"(acc[nt][mt - 1]));  // keeps the promotion here, in the shadow of the MFMAs above
-          }
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if constexpr (!MX) {
-#pragma unroll
-      for (int nt = 0; nt < NTW; nt++) {
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-          acc[nt][MTW - 1][i] = __builtin_fmaf(tmp[(MTW - 1) & 1][nt][i], f.sc[MTW - 1] * ((FUSE && nt >= NTW / 2) ? f.sb_up : f.sb), acc[nt][MTW - 1][i]);
-        asm volatile("" : "+v"(acc[nt][MTW - 1]));
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
@@ -658,14 +622,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   // kb+1; for mxfp8 the weight rows a phase later, see kSplitIssue).  Issuing copies costs a wavefront
   // a few hundred cycles in the queue to the texture path, so where they sit decides which phase is
   // the longer one.
-  // Tiles whose mfma phase still reads token fragments from LDS (16 row tiles per wavefront do not
-  // fit in registers) run both groups in step, with no barrier between the phases.
-  // Measured per tile height on dense problems: the two-group alternation pays for fp8-blockwise tiles of 128 and
-  // 192 rows and mxfp8 tiles of 192 rows; the short tiles (and 128-row mxfp8 tiles) run 4-14 % faster with all
-  // eight wavefronts in step (bit i of the mask: height index i of {16, 32, 64, 128, 192, 256} rows in step).
-  constexpr int kHeightIdx = MT == 1 ? 0 : MT == 2 ? 1 : MT == 4 ? 2 : MT == 8 ? 3 : MT == 12 ? 4 : 5;
-  constexpr int kInStepMask = MX ? 0b001100 : 0b000111;
-  constexpr bool kPP = kPre == MTW && !((kInStepMask >> kHeightIdx) & 1);
+  // Measured per tile height on dense problems: the short fp8-blockwise tiles and the 64-row mxfp8 tile run 4-14 %
+  // faster with all eight wavefronts in step (no barrier between the phases); the 16- and 32-row mxfp8 tiles alternate.
+  constexpr bool kPP = MX && MT < 4;
   const int grp = kPP ? wave >> 2 : 0;
   // mxfp8 (no vector-ALU work in the mfma phase): token copies go out in the read phase, weight copies in
   // the mfma phase.  fp8-blockwise: the mfma phase is already the longer one with its promotions, so
@@ -706,7 +665,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       else if (kb + NBUF < KB) issue_w(kb + NBUF, buf);
     }
     __builtin_amdgcn_sched_barrier(0);
-    mfma_phase(buf, f);
+    mfma_phase(f);
     __builtin_amdgcn_sched_barrier(0);
     if (grp == 0) wait_stage(more, chunk_age < NBUF - 2);
     chunk_age++;
