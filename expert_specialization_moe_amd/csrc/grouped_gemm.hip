@@ -481,9 +481,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 #pragma unroll
     for (int mt = 0; mt < MTW; mt++) acc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  // The work on one K block is split in two phases, so that the two groups of four wavefronts (one
-  // wavefront of each group per SIMD) can run half an iteration apart: while one group's MFMAs keep
-  // the matrix pipe busy, the other group reads its fragments from LDS.
+  // The work on one K block is split in two phases:
   //   read phase: weight fragments, token fragments and all scales -> registers (every fragment of a short tile fits)
   //   mfma phase: the MFMAs (+ the fp32 promotion for fp8-blockwise) of the K block
   struct Frags {
@@ -615,21 +613,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   else wait_vmcnt<(NBUF - 2) * G::kCopiesPerStage>();
   block_barrier();
 
-  // Barrier intervals alternate; group 0 (wavefronts 0-3) reads K block kb in interval 2kb and runs its
-  // MFMAs in interval 2kb+1, group 1 (wavefronts 4-7) does each one interval later.  Ring slot of K
-  // block kb is therefore read during intervals 2kb and 2kb+1 and must be complete before interval
-  // 2kb starts; it is refilled with K block kb+NBUF from interval 2kb+2 on (each group's read phase
-  // kb+1; for mxfp8 the weight rows a phase later, see kSplitIssue).  Issuing copies costs a wavefront
-  // a few hundred cycles in the queue to the texture path, so where they sit decides which phase is
-  // the longer one.
-  // Measured per tile height on dense problems: the short fp8-blockwise tiles and the 64-row mxfp8 tile run 4-14 %
-  // faster with all eight wavefronts in step (no barrier between the phases); the 16- and 32-row mxfp8 tiles alternate.
-  constexpr bool kPP = MX && MT < 4;
-  const int grp = kPP ? wave >> 2 : 0;
-  // mxfp8 (no vector-ALU work in the mfma phase): token copies go out in the read phase, weight copies in
-  // the mfma phase.  fp8-blockwise: the mfma phase is already the longer one with its promotions, so
-  // the read phase issues the whole stage.
-  constexpr bool kSplitIssue = kPP && MX;
+  // All eight wavefronts run in step, one barrier per K block: the stage of K block kb + NBUF - 1 is requested at the
+  // top of iteration kb into the slot that iteration kb - 1 read.  (Two groups of wavefronts half an iteration apart, as in
+  // the tall tiles, were measured for every short height and both kernels: 0.2-14 % slower; a short tile is bound by its
+  // weight stream, not by the overlap of reads and MFMAs.)
   auto wait_stage = [&](bool more, int chunk_young) {
     // all of this wavefront's copies except those of the newest NBUF-2 K blocks have landed
     if (!more) wait_vmcnt<0>();
@@ -639,10 +626,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   };
   int buf = 0, nbuf = NBUF - 1;  // ring slots of K block kb and of K block kb + NBUF - 1
   int chunk_age = NBUF;          // iterations since this wavefront issued a scale-chunk copy
-  if (grp == 1) {
-    if constexpr (kSplitIssue) { if (NBUF - 1 < KB) issue_w(NBUF - 1, nbuf); }
-    block_barrier();
-  }
   Frags f;
   for (int kb = 0; kb < KB; kb++) {
     const bool more = kb + NBUF - 1 < KB;
@@ -654,26 +637,18 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
       chunk_age = 0;
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (more) { if constexpr (kSplitIssue) issue_a(kb + NBUF - 1, nbuf); else issue(kb + NBUF - 1, nbuf); }
+    if (more) issue(kb + NBUF - 1, nbuf);
     __builtin_amdgcn_sched_barrier(0);
     read_phase(kb, buf, f);
     __builtin_amdgcn_sched_barrier(0);
-    if (grp == 1) wait_stage(more, chunk_age < NBUF - 2);
-    if constexpr (kPP) block_barrier();
-    if constexpr (kSplitIssue) {
-      if (grp == 0) { if (more) issue_w(kb + NBUF - 1, nbuf); }
-      else if (kb + NBUF < KB) issue_w(kb + NBUF, buf);
-    }
-    __builtin_amdgcn_sched_barrier(0);
     mfma_phase(f);
     __builtin_amdgcn_sched_barrier(0);
-    if (grp == 0) wait_stage(more, chunk_age < NBUF - 2);
+    wait_stage(more, chunk_age < NBUF - 2);
     chunk_age++;
     block_barrier();
     buf = buf + 1 == NBUF ? 0 : buf + 1;
     nbuf = nbuf + 1 == NBUF ? 0 : nbuf + 1;
   }
-  if (kPP && grp == 0) block_barrier();
 
   if constexpr (MX && FUSE) tile_epilogue_mxq<G::BM, MTW, NTW, G::kWavesN>(g, acc, e, M, m0, n0, row_base, mw, wn, lane, lds);
   else tile_epilogue<G::BM, MTW, NTW, G::kWavesN, FUSE>(g, acc, M, m0, n0, row_base, mw, nw, wn, lane, wave_active, lds);
