@@ -20,9 +20,9 @@ import torch
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "gemm"): 1.547e9,     # FETCH 728,528.8 x 2.000 KiB + WRITE 53,264.5 x 1.000 KiB
-    ("c2", "gemm"): 4.490e8,     # FETCH 217,422.8 x 2.000 KiB + WRITE 3,631.8 x 1.000 KiB
-    ("c4", "gemm"): 1.456e9,     # FETCH 677,983.3 x 2.000 KiB + WRITE 66,257.2 x 1.000 KiB
+    ("c1", "gemm"): 1.576e9,     # FETCH 742,662.6 x 2.000 KiB + WRITE 53,284.9 x 1.000 KiB
+    ("c2", "gemm"): 4.488e8,     # FETCH 217,330.2 x 2.000 KiB + WRITE 3,631.5 x 1.000 KiB
+    ("c4", "gemm"): 1.456e9,     # FETCH 677,579.2 x 2.000 KiB + WRITE 66,249.9 x 1.000 KiB
     ("c4", "quant"): 1.786e8,    # FETCH 57,399.0 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
 }
 
