@@ -185,7 +185,7 @@ def emit(name, mtw, fuse):
 
 # ---- mxfp8 form ----------------------------------------------------------------------------------------------------
 # Same ring and phases with the hardware-scaled MFMA accumulating straight into the accumulators: no promotions, no
-# result buffers.  The E8M0 scale bytes travel with the stages as verbatim 512-byte scale tiles (2 for the weight
+# result buffers, and the K loop's bookkeeping inside the statement (mx_bookkeeping).  The E8M0 scale bytes travel with the stages as verbatim 512-byte scale tiles (2 for the weight
 # rows behind a weight stage, 2 for the group's token rows behind its token stage); every wavefront issues one
 # 1 KB scale copy per K block so that the counted waits are the same for all (wavefront 0: weight scales of K block
 # kb + 2, wavefronts 1 and 5: their group's token scales of kb + 1, the others re-read one line into a spare area).
@@ -202,7 +202,7 @@ class MxPlan:
         self.ntc = mtw // 2
 
     def clobbers(self):
-        return [f'"v{i}"' for i in range(self.lowest, 256)] + ['"memory"', '"m0"']
+        return [f'"v{i}"' for i in range(self.lowest, 256)] + ['"memory"', '"m0"', '"scc"', '"vcc"']
 
 
 def mx_memory_phase(p):
@@ -248,9 +248,44 @@ def mx_memory_phase(p):
     return L
 
 
+def mx_bookkeeping(p):
+    """What changes from one K block to the next, advanced inside the statement: the lines sit behind the MFMAs of the
+    matrix phase, where the wavefront has issue slots to spare, instead of between two statements, where they would
+    delay the copies of the next memory phase (the critical path of a K block, the other group's MFMAs running beside
+    it).  Every operand the memory phase uses is an in/out operand that holds the value for the coming K block:
+
+        token slot (2-cycle)    %[td] = +-(bytes of a token slot): la -= td; al, sfa* += td; ah = al ^ 64; td = -td
+        weight slot (3-cycle)   lw += S, back to %[lwbase] at %[lwend]; %[woff] in {0, S, 2S}: wl = wfrag + woff, wh = wl ^ 64,
+                                sfwl = sfwrd + woff
+        scale copy target       ls += %[lsinc], minus %[lswrap] at %[lsend] (the three roles differ in these constants only)
+        copy sources            the lanes' byte offsets advance (the base pointers stay): by 128 (512 for the scale tiles)
+                                while a later K block exists, counted down in %[rem] (K blocks after this one)
+
+    Returns groups of lines; a group stays together (its s_cmp / s_cselect pair shares SCC with nothing else)."""
+    S = 256 * 128 + 1024
+    A = []
+    A.append(["s_sub_u32 %[la], %[la], %[td]"])
+    for mt in range(p.mtw):
+        A.append([f"v_add_u32 %[sfa{mt}], %[td], %[sfa{mt}]"])
+    A.append([f"s_add_u32 %[lw], %[lw], {S}", "s_cmp_lg_u32 %[lw], %[lwend]", "s_cselect_b32 %[lw], %[lw], %[lwbase]"])
+    A.append([f"s_add_u32 %[woff], %[woff], {S}", f"s_cmp_lg_u32 %[woff], {3 * S}", "s_cselect_b32 %[woff], %[woff], 0"])
+    A.append(["v_add_u32 %[wl], %[woff], %[wfrag]", "v_xor_b32 %[wh], 64, %[wl]", "v_add_u32 %[sfwl], %[woff], %[sfwrd]"])
+    A.append(["s_add_u32 %[ls], %[ls], %[lsinc]", "s_cmp_ge_u32 %[ls], %[lsend]", "s_cselect_b32 vcc_lo, %[lswrap], 0",
+              "s_sub_u32 %[ls], %[ls], vcc_lo"])
+    A.append(["s_cmp_ge_u32 %[rem], 2", "s_cselect_b32 vcc_lo, 128, 0"] + [f"v_add_u32 %[va{i}], vcc_lo, %[va{i}]" for i in range(p.ntc)])
+    A.append(["s_cmp_ge_u32 %[rem], 3", "s_cselect_b32 vcc_lo, 128, 0"] + [f"v_add_u32 %[vw{i}], vcc_lo, %[vw{i}]" for i in range(4)])
+    A.append(["s_cmp_ge_u32 %[rem], %[sthr]", "s_cselect_b32 vcc_lo, 0x200, 0", "v_add_u32 %[vs], vcc_lo, %[vs]", "s_sub_u32 %[rem], %[rem], 1"])
+    # after the last rolling token read (it still uses al, ah), and td's sign flips last
+    late = [["v_add_u32 %[al], %[td], %[al]", "v_xor_b32 %[ah], 64, %[al]"], ["s_sub_u32 %[td], 0, %[td]"]]
+    return A, late
+
+
 def mx_matrix_phase(p):
     L = []
-    for j in range(p.mtw * NT):
+    atoms, late = mx_bookkeeping(p) if "nobook" not in ABLATE else ([], [])
+    total = p.mtw * NT
+    last_roll = (p.mtw - 3) * NT      # MFMA behind which the last rolling token read issues
+    for j in range(total):
         mt, nt = divmod(j, NT)
         if nt == 0 and mt >= 2:
             L.append("s_waitcnt lgkmcnt(2)" if mt + 1 < p.mtw else "s_waitcnt lgkmcnt(0)")
@@ -260,6 +295,12 @@ def mx_matrix_phase(p):
             b = p.a[(mt + 2) % 3]
             L.append(f"ds_read_b128 {regs(b, 4)}, %[al] offset:{(mt + 2) * 2048}")
             L.append(f"ds_read_b128 {regs(b + 4, 4)}, %[ah] offset:{(mt + 2) * 2048}")
+        # one group of bookkeeping behind each of the first MFMAs; the token-slot group once al and ah are free
+        if j >= 1 and atoms:
+            L += atoms.pop(0)
+        if j > last_roll and not atoms and late:
+            L += late.pop(0)
+    assert not atoms and not late, "more bookkeeping than MFMAs"
     L.append("s_waitcnt vmcnt(4) ; explicit")
     L.append("s_barrier")
     return L
@@ -269,11 +310,15 @@ def emit_mx(name, mtw, fuse=False):
     p = MxPlan(mtw, fuse)
     lines = ablated(mx_memory_phase(p) + mx_matrix_phase(p))
     print_body(name, lines)
-    print(f"#define {name}_OUTS " + ", ".join(f'[c{nt}_{mt}] "+v"(acc[{nt}][{mt}])' for mt in range(mtw) for nt in range(NT)))
-    ins = [f'[va{i}] "v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "v"(vw[{i}])' for i in range(4)]
-    ins += ['[vs] "v"(vs)', '[wl] "v"(wl)', '[wh] "v"(wh)', '[al] "v"(al)', '[ah] "v"(ah)', '[sfwl] "v"(sfwl)']
-    ins += [f'[sfa{mt}] "v"(sfal[{mt}])' for mt in range(mtw)]
-    ins += ['[sh] "v"(shift)', '[la] "s"(la)', '[lw] "s"(lw)', '[ls] "s"(ls)', '[ap] "s"(ap)', '[wp] "s"(wp)', '[sp] "s"(sp)']
+    outs = [f'[c{nt}_{mt}] "+v"(acc[{nt}][{mt}])' for mt in range(mtw) for nt in range(NT)]
+    outs += [f'[va{i}] "+v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "+v"(vw[{i}])' for i in range(4)]
+    outs += ['[vs] "+v"(vs)', '[wl] "+v"(wl)', '[wh] "+v"(wh)', '[al] "+v"(al)', '[ah] "+v"(ah)', '[sfwl] "+v"(sfwl)']
+    outs += [f'[sfa{mt}] "+v"(sfal[{mt}])' for mt in range(mtw)]
+    outs += ['[la] "+s"(la)', '[lw] "+s"(lw)', '[ls] "+s"(ls)', '[td] "+s"(td)', '[woff] "+s"(woff)', '[rem] "+s"(rem)']
+    print(f"#define {name}_OUTS " + ", ".join(outs))
+    ins = ['[wfrag] "v"(wfrag)', '[sfwrd] "v"(sfw_rd)', '[sh] "v"(shift)', '[ap] "s"(a_ptr)', '[wp] "s"(w_ptr)', '[sp] "s"(s_ptr)',
+           '[lwbase] "s"(lwbase)', '[lwend] "s"(lwend)', '[lsinc] "s"(lsinc)', '[lsend] "s"(lsend)', '[lswrap] "s"(lswrap)',
+           '[sthr] "s"(sthr)']
     print(f"#define {name}_INS " + ", ".join(ins))
     print(f"#define {name}_CLOBBERS " + ", ".join(p.clobbers()))
     print(f"#define {name}_LOWEST_FIXED_VGPR {p.lowest}")

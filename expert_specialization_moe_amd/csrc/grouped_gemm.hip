@@ -959,29 +959,35 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
   const uint64_t tl_r0 = __builtin_amdgcn_s_memrealtime(), tl_c0 = __builtin_amdgcn_s_memtime();
 #endif
   const bool w_once = ESMOE_PP_NT && m0 == 0 && M <= BM;   // nobody else reads these weight rows: non-temporal copies (see gemm_tile_pp)
+  // Everything that changes from one K block to the next is an in/out operand of the statement, which advances it
+  // behind its MFMAs (gen_pp_phase.py, mx_bookkeeping); the values below are those of K block 0: token slot 0 is
+  // read and slot 1 filled, weight slot 0 is read and slot 2 filled, the copies fetch token stage 1 and weight stage 2.
+  uint32_t la = t_dst + kTSlot, td = kTSlot;
+  uint32_t lw = w_dst + 2 * kWSlot, woff = 0;
+  const uint32_t lwbase = w_dst, lwend = w_dst + 3 * kWSlot;
+  uint32_t ls = s_dst + (s_role == 0 ? 2 * kWSlot : s_role == 1 ? kTSlot : 0);
+  const uint32_t lsinc = s_role == 0 ? kWSlot : s_role == 1 ? kTSlot : 0;
+  const uint32_t lsend = s_role == 0 ? s_dst + 3 * kWSlot : s_role == 1 ? s_dst + 2 * kTSlot : 0xffffffffu;
+  const uint32_t lswrap = s_role == 0 ? 3 * kWSlot : s_role == 1 ? 2 * kTSlot : 0;
+  const uint32_t sthr = s_role == 0 ? 3 : 2;   // the scale copy goes with the weight stage (two K blocks ahead) or the token stage (one)
+  uint32_t rem = KB - 1;                       // K blocks after the one at hand
+  const int kbt0 = 1 < KB ? 1 : KB - 1, kbw0 = 2 < KB ? 2 : KB - 1;
+#pragma unroll
+  for (int i = 0; i < kTCopies; i++) va[i] += kbt0 * 128;
+#pragma unroll
+  for (int i = 0; i < 4; i++) vw[i] += kbw0 * 128;
+  vs += (s_role == 0 ? kbw0 : kbt0) * 512;
+  uint32_t wl = wfrag, wh = wfrag ^ 64, al = afrag, ah = afrag ^ 64, sfwl = sfw_rd;
+  uint32_t sfal[MTW];
+#pragma unroll
+  for (int mt = 0; mt < MTW; mt++) sfal[mt] = sfa_rd[mt];
   auto k_loop = [&](auto nt_hint) {
     constexpr bool kNt = decltype(nt_hint)::value;
-    int tslot = 0, wslot = 0;
     for (int kb = 0; kb < KB; kb++) {
-      const int kbt = kb + 1 < KB ? kb + 1 : KB - 1, kbw = kb + 2 < KB ? kb + 2 : KB - 1;
-      const int wnext = wslot >= 1 ? wslot - 1 : 2;          // (kb + 2) % 3
-      const uint32_t la = t_dst + (tslot ^ 1) * kTSlot, lw = w_dst + wnext * kWSlot;
-      const uint32_t ls = s_dst + (s_role == 0 ? wnext * kWSlot : s_role == 1 ? (tslot ^ 1) * kTSlot : 0);
-      const uint8_t* ap = a_ptr + (long)kbt * 128;
-      const uint8_t* wp = w_ptr + (long)kbw * 128;
-      const uint8_t* sp = s_ptr + (long)(s_role == 0 ? kbw : kbt) * 512;
-      const uint32_t wl = wfrag + wslot * kWSlot, wh = wl ^ 64;
-      const uint32_t al = afrag + tslot * kTSlot, ah = al ^ 64;
-      const uint32_t sfwl = sfw_rd + wslot * kWSlot;
-      uint32_t sfal[MTW];
-#pragma unroll
-      for (int mt = 0; mt < MTW; mt++) sfal[mt] = sfa_rd[mt] + tslot * kTSlot;
       if constexpr (MT == 12 && FUSE) ESMOE_PP_STMT(ESMOE_PPX12F);
       else if constexpr (MT == 12) ESMOE_PP_STMT(ESMOE_PPX12);
       else if constexpr (FUSE) ESMOE_PP_STMT(ESMOE_PPX8F);
       else ESMOE_PP_STMT(ESMOE_PPX8);
-      tslot ^= 1;
-      wslot = wslot == 2 ? 0 : wslot + 1;
     }
   };
   if (w_once) k_loop(std::true_type{}); else k_loop(std::false_type{});
