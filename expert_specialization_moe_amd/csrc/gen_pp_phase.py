@@ -14,6 +14,10 @@ run half a K block apart.  A K block of a wavefront is
     s_barrier
     the last three promotions (in the shadow of the other group's first MFMAs)
 
+and the statement also advances, behind its first three MFMAs (which have no promotions to issue yet), what changes from
+one K block to the next of token slot, weight slot and copy sources (bookkeeping): between two statements those
+instructions would delay the next memory phase's copies.
+
 so while one group's wavefront keeps its SIMD's matrix pipe busy, the other group's wavefront on that SIMD moves data.
 Written as a statement, not as C++ with scheduling fences: the compiler neither keeps such an order nor tracks the
 asynchronous copies (its own waits would land in the loop), and every register that lives only inside the K block
@@ -36,7 +40,8 @@ a write of m0 from the copy that uses it.
 import sys
 
 NT = 4
-ABLATE = set()   # timing experiments only (results wrong): "fma", "copy", "roll", "read", "barrier", "vmwait"
+ABLATE = set()   # timing experiments only (results wrong): "fma", "copy", "roll", "read", "barrier", "vmwait";
+                 # "bookodd": bookkeeping behind every second MFMA instead (results right)
 
 
 def regs(lo, n):
@@ -58,7 +63,7 @@ class Plan:
         self.ntc = mtw // 2                               # token copies per wavefront and K block
 
     def clobbers(self):
-        return [f'"v{i}"' for i in range(self.lowest, 256)] + ['"memory"', '"m0"']
+        return [f'"v{i}"' for i in range(self.lowest, 256)] + ['"memory"', '"m0"', '"scc"', '"vcc"']
 
 
 def memory_phase(p):
@@ -111,10 +116,29 @@ def promotion(p, j):
     return [f"v_fmac_f32 %[c{nt}_{mt}_{i}], v{p.t[j % 4] + i}, v{sc}" for i in range(4)]
 
 
+def bookkeeping(p):
+    """The part of the K loop's bookkeeping that this statement advances itself, behind its MFMAs (see mx_bookkeeping
+    for the scheme and the reason): token slot, weight slot and the copies' source offsets.  What goes with the scale
+    chunks (a four-K-block rhythm with an irregular last chunk) stays with the caller."""
+    S = 256 * 128
+    A = []
+    A.append(["s_sub_u32 %[la], %[la], %[td]"])
+    A.append([f"s_add_u32 %[lw], %[lw], {S}", "s_cmp_lg_u32 %[lw], %[lwend]", "s_cselect_b32 %[lw], %[lw], %[lwbase]"])
+    A.append([f"s_add_u32 %[woff], %[woff], {S}", f"s_cmp_lg_u32 %[woff], {3 * S}", "s_cselect_b32 %[woff], %[woff], 0"])
+    A.append(["v_add_u32 %[wl], %[woff], %[wfrag]", "v_xor_b32 %[wh], 64, %[wl]"])
+    A.append(["s_cmp_ge_u32 %[rem], 2", "s_cselect_b32 vcc_lo, 128, 0"] + [f"v_add_u32 %[va{i}], vcc_lo, %[va{i}]" for i in range(p.ntc)])
+    A.append(["s_cmp_ge_u32 %[rem], 3", "s_cselect_b32 vcc_lo, 128, 0"] + [f"v_add_u32 %[vw{i}], vcc_lo, %[vw{i}]" for i in range(4)]
+             + ["s_sub_u32 %[rem], %[rem], 1"])
+    late = [["v_add_u32 %[al], %[td], %[al]", "v_xor_b32 %[ah], 64, %[al]"], ["s_sub_u32 %[td], 0, %[td]"]]
+    return A, late
+
+
 def matrix_phase(p):
     L = []
     total = p.mtw * NT
     lag = 3
+    atoms, late = bookkeeping(p) if "nobook" not in ABLATE else ([], [])
+    last_roll = (p.mtw - 3) * NT      # MFMA behind which the last rolling token read issues
     for j in range(total):
         mt, nt = divmod(j, NT)
         if nt == 0 and mt >= 2:
@@ -126,6 +150,18 @@ def matrix_phase(p):
             L.append(f"ds_read_b128 {regs(b + 4, 4)}, %[ah] offset:{(mt + 2) * 2048}")
         if j >= lag:
             L += promotion(p, j - lag)
+        # bookkeeping behind the first three MFMAs, which have no promotions to issue yet (two groups each); the
+        # token-slot group once the last rolling read has used al and ah
+        if "bookodd" in ABLATE:
+            if j >= 1 and atoms and j % 2 == 1:
+                L += atoms.pop(0)
+        elif j < lag:
+            for _ in range(2):
+                if atoms:
+                    L += atoms.pop(0)
+        if j > last_roll and not atoms and late:
+            L += late.pop(0)
+    assert not atoms and not late, "more bookkeeping than MFMAs"
     L.append("s_waitcnt vmcnt(4) ; explicit")
     L.append("s_barrier")
     for j in range(total - lag, total):
@@ -173,11 +209,13 @@ def emit(name, mtw, fuse):
     p = Plan(mtw, fuse)
     lines = ablated(memory_phase(p) + matrix_phase(p))
     print_body(name, lines)
-    print(f"#define {name}_OUTS " + ", ".join(
-        f'[c{nt}_{mt}_{i}] "+v"(acc[{nt}][{mt}][{i}])' for mt in range(mtw) for nt in range(NT) for i in range(4)))
-    ins = [f'[va{i}] "v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "v"(vw[{i}])' for i in range(4)]
-    ins += ['[vs] "v"(vsq)', '[wl] "v"(wl)', '[wh] "v"(wh)', '[al] "v"(al)', '[ah] "v"(ah)', '[sal] "v"(sal)', '[sbl] "v"(sbl)',
-            '[la] "s"(la)', '[lw] "s"(lw)', '[ls] "s"(ls)', '[ap] "s"(ap)', '[wp] "s"(wp)', '[sp] "s"(sp)']
+    outs = [f'[c{nt}_{mt}_{i}] "+v"(acc[{nt}][{mt}][{i}])' for mt in range(mtw) for nt in range(NT) for i in range(4)]
+    outs += [f'[va{i}] "+v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "+v"(vw[{i}])' for i in range(4)]
+    outs += ['[wl] "+v"(wl)', '[wh] "+v"(wh)', '[al] "+v"(al)', '[ah] "+v"(ah)']
+    outs += ['[la] "+s"(la)', '[lw] "+s"(lw)', '[td] "+s"(td)', '[woff] "+s"(woff)', '[rem] "+s"(rem)']
+    print(f"#define {name}_OUTS " + ", ".join(outs))
+    ins = ['[vs] "v"(vsq)', '[sal] "v"(sal)', '[sbl] "v"(sbl)', '[wfrag] "v"(wfrag)',
+           '[ls] "s"(ls)', '[ap] "s"(a_ptr)', '[wp] "s"(w_ptr)', '[sp] "s"(sp)', '[lwbase] "s"(lwbase)', '[lwend] "s"(lwend)']
     print(f"#define {name}_INS " + ", ".join(ins))
     print(f"#define {name}_CLOBBERS " + ", ".join(p.clobbers()))
     print(f"#define {name}_LOWEST_FIXED_VGPR {p.lowest}")

@@ -781,22 +781,31 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
   // that their stream leaves L2 to the operands that are shared.  One loop per form: a statement of each kind on
   // alternative paths of one loop would make the compiler shuffle the accumulators between them.
   const bool w_once = ESMOE_PP_NT && m0 == 0 && M <= BM;
+  // The token slot, the weight slot and the copies' source offsets are in/out operands of the statement, which advances
+  // them behind its MFMAs (gen_pp_phase.py, bookkeeping); the values below are those of K block 0: token slot 0 is read
+  // and slot 1 filled, weight slot 0 is read and slot 2 filled, the copies fetch token stage 1 and weight stage 2.  What
+  // goes with the scale chunks stays here.
+  uint32_t la = t_dst + kTSlot, td = kTSlot;
+  uint32_t lw = w_dst + 2 * kWSlot, woff = 0;
+  const uint32_t lwbase = w_dst, lwend = w_dst + 3 * kWSlot;
+  uint32_t rem = KB - 1;                       // K blocks after the one at hand
+  {
+    const int kbt0 = 1 < KB ? 1 : KB - 1, kbw0 = 2 < KB ? 2 : KB - 1;
+#pragma unroll
+    for (int i = 0; i < kTCopies; i++) va[i] += kbt0 * 128;
+#pragma unroll
+    for (int i = 0; i < 4; i++) vw[i] += kbw0 * 128;
+  }
+  uint32_t wl = wfrag, wh = wfrag ^ 64, al = afrag, ah = afrag ^ 64;
   auto k_loop = [&](auto nt_hint) {
     constexpr bool kNt = decltype(nt_hint)::value;
-    int tslot = 0, wslot = 0, sabuf = 0;   // slots of K block kb: tokens kb % 2, weights kb % 3, scale chunk (kb / 4) % 3
+    int sabuf = 0;   // buffer of the scale chunk of K block kb: (kb / 4) % 3
     for (int kb = 0; kb < KB; kb++) {
       const int q = kb & 3;
-      const int kbt = kb + 1 < KB ? kb + 1 : KB - 1, kbw = kb + 2 < KB ? kb + 2 : KB - 1;
       const int chw = (kb >> 2) + 2 < NCH ? (kb >> 2) + 2 : NCH - 1;
-      const int wnext = wslot >= 1 ? wslot - 1 : 2;          // (kb + 2) % 3
       const int sanext = sabuf >= 1 ? sabuf - 1 : 2;         // (kb / 4 + 2) % 3
-      const uint32_t la = t_dst + (tslot ^ 1) * kTSlot, lw = w_dst + wnext * kWSlot;
       const uint32_t ls = s_dst + sanext * kSaBuf + q * 256;
-      const uint8_t* ap = a_ptr + (long)kbt * 128;
-      const uint8_t* wp = w_ptr + (long)kbw * 128;
       const uint8_t* sp = sa_ptr + (long)chunk_first_kb(chw) * 4;
-      const uint32_t wl = wfrag + wslot * kWSlot, wh = wl ^ 64;
-      const uint32_t al = afrag + tslot * kTSlot, ah = al ^ 64;
       const uint32_t sal = sa_rd + sabuf * kSaBuf + (kb - chunk_first_kb(kb >> 2)) * 4;
       const uint32_t sbl = sb_rd + kb * 4;
       const uint32_t vsq = vs[0];
@@ -809,10 +818,8 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
       else if constexpr (MT == 12) ESMOE_PP_STMT(ESMOE_PP12);
       else if constexpr (FUSE) ESMOE_PP_STMT(ESMOE_PP8F);
       else ESMOE_PP_STMT(ESMOE_PP8);
-      // the piece offsets rotate with q; slots advance
+      // the piece offsets rotate with q; the chunk buffer advances every fourth K block
       { const uint32_t t = vs[0]; vs[0] = vs[1]; vs[1] = vs[2]; vs[2] = vs[3]; vs[3] = t; }
-      tslot ^= 1;
-      wslot = wslot == 2 ? 0 : wslot + 1;
       if (q == 3) sabuf = sabuf == 2 ? 0 : sabuf + 1;
     }
   };
