@@ -130,6 +130,11 @@ __device__ __forceinline__ int sload(const int* base, int byte_offset) {
   asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(base), "s"(__builtin_amdgcn_readfirstlane(byte_offset)) : "memory");
   return __builtin_amdgcn_readfirstlane(v);
 }
+__device__ __forceinline__ v4i sload4(const int* base, int byte_offset) {   // 16 bytes, 16-byte aligned
+  v4i v;
+  asm volatile("s_load_dwordx4 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(base), "s"(__builtin_amdgcn_readfirstlane(byte_offset)) : "memory");
+  return v;
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0) ; explicit" ::"n"(N) : "memory");
@@ -269,7 +274,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, Acc& acc, int M
 // their maxima through LDS.  Scale bytes of the rows between the expert's last row and the end of its last 128-row
 // scale tile are written as 0, as the stand-alone quantisation does.
 template <int BM, int MTW, int NTW, int kWavesN, typename Acc>
-__device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, int e, int M, int m0, int n0,
+__device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, int ebso, int M, int m0, int n0,
                                                   long row_base, int mw, int wn, int lane, uint8_t* lds) {
   constexpr int kHalf = NTW / 2, kRW = NTW * 16;
   constexpr bool kPair = kHalf == 1;
@@ -306,7 +311,7 @@ __device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, i
     if (kPair && gq == 0) s_amax[wn * BM + mw + mt * 16 + r] = amax;
   }
   if constexpr (kPair) __syncthreads();
-  uint8_t* sf_e = g.sf_out + (long)g.blockscale_offsets[e] * (inter >> 5);
+  uint8_t* sf_e = g.sf_out + (long)ebso * (inter >> 5);
   const int cblk = (n0 >> 6) + ((wn * (kRW / 2)) >> 5);   // 32-column block of this wavefront's h columns
   const int m_pad = (M + 127) & ~127;
 #pragma unroll
@@ -348,7 +353,7 @@ __device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, i
 // epilogue forms silu(gate) * up and quantises it for the down projection (fp8-blockwise: 1x128 blocks with fp32
 // scales, tile_epilogue; mxfp8: 1x32 blocks with E8M0 scales, tile_epilogue_mxq) instead of writing the projection.
 template <int MT, bool MX, bool FUSE, int BN = kBN>
-__device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds) {
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int erow, int ebso, int M, int m0, int n0, uint8_t* lds) {
   static_assert(!(FUSE && BN != kBN), "the fused epilogues need gate and up columns of a whole quantisation block in one tile");
   static_assert(MT == 1 || MT == 2 || MT == 4, "short tiles; 128- and 192-row tiles are gemm_tile_pp / gemm_tile_pp_mx");
   using G = TileGeom<MT, MX, BN>;
@@ -360,7 +365,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
   const int r = lane & 15;
   const int gq = lane >> 4;
   const int K = g.k, N = g.n, KB = K >> 7;
-  const long row_base = g.expert_offsets[e];
+  const long row_base = erow;
   const int nw = wn * (NTW * 16);          // first weight row of this wavefront inside the tile
   const int mw = wm * (MTW * 16);          // first token row of this wavefront inside the tile
   const bool wave_active = n0 + nw < N;
@@ -402,7 +407,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     } else {                // odd wavefronts: the token scale tile(s)
       blk = (m0 >> 7) + (lane >> 5);
       if (blk * 128 >= M) blk = m0 >> 7;
-      sc_base = g.sfa + (long)g.blockscale_offsets[e] * kc;
+      sc_base = g.sfa + (long)ebso * kc;
     }
     scoff = (uint32_t)blk * (uint32_t)KB * 512 + (lane & 31) * 16;
     sclds = G::kABytes + G::kWBytes + (wave & 1) * 1024;
@@ -650,7 +655,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
     nbuf = nbuf + 1 == NBUF ? 0 : nbuf + 1;
   }
 
-  if constexpr (MX && FUSE) tile_epilogue_mxq<G::BM, MTW, NTW, G::kWavesN>(g, acc, e, M, m0, n0, row_base, mw, wn, lane, lds);
+  if constexpr (MX && FUSE) tile_epilogue_mxq<G::BM, MTW, NTW, G::kWavesN>(g, acc, ebso, M, m0, n0, row_base, mw, wn, lane, lds);
   else tile_epilogue<G::BM, MTW, NTW, G::kWavesN, FUSE>(g, acc, M, m0, n0, row_base, mw, nw, wn, lane, wave_active, lds);
 }
 
@@ -670,7 +675,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int M, int m
 // slot is refilled with stage kb + 3 from 2kb + 2 on, three or more intervals before 2kb + 6; a group's token stage
 // kb is read in its memory and matrix phase of kb and refilled in its memory phase of kb + 1 with stage kb + 2.
 template <int MT, bool FUSE>
-__device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds,
+__device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int erow, int M, int m0, int n0, uint8_t* lds,
                                              uint32_t* timeline = nullptr) {
   static_assert(MT == 8 || MT == 12, "hand-scheduled K block: 128- and 192-row tiles");
   constexpr int MTW = MT / 2, NTW = 4, BM = MT * 16, GR = MTW * 16;
@@ -687,7 +692,7 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
   // a K that is no multiple of 512 overlaps the one before instead of reaching past the row.
   const int K = g.k, N = g.n, KB = K >> 7, NCH = (KB + 3) >> 2;
   auto chunk_first_kb = [&](int c) { const int f = 4 * c < KB - 4 ? 4 * c : KB - 4; return f > 0 ? f : 0; };
-  const long row_base = g.expert_offsets[e];
+  const long row_base = erow;
   const int nw = wj * 64, mw = grp * GR;
   const bool wave_active = n0 + nw < N;
   const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
@@ -847,7 +852,7 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int M, in
 // A tile may start in the middle of a 128-row scale tile (full tiles are 192 rows): a lane finds the scale dword of
 // its row from the row's position inside the two tiles that were fetched for its group.
 template <int MT, bool FUSE>
-__device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M, int m0, int n0, uint8_t* lds,
+__device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int erow, int ebso, int M, int m0, int n0, uint8_t* lds,
                                                 uint32_t* timeline = nullptr) {
   static_assert(MT == 8 || MT == 12, "hand-scheduled K block: 128- and 192-row tiles");
   constexpr int MTW = MT / 2, NTW = 4, BM = MT * 16, GR = MTW * 16;
@@ -861,7 +866,7 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
   const int grp = wave >> 2, wj = wave & 3;
   const int r = lane & 15, gq = lane >> 4;
   const int K = g.k, N = g.n, KB = K >> 7, kc = K >> 5;
-  const long row_base = g.expert_offsets[e];
+  const long row_base = erow;
   const int nw = wj * 64, mw = grp * GR;
   const bool wave_active = n0 + nw < N;
   const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
@@ -911,7 +916,7 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
   } else if (s_role == 1) {
     int blk = tblk0 + (lane >> 5);
     if (blk * 128 >= M) blk = tblk0 * 128 < M ? tblk0 : m0 >> 7;
-    s_ptr = g.sfa + (long)g.blockscale_offsets[e] * kc;
+    s_ptr = g.sfa + (long)ebso * kc;
     vs = (uint32_t)blk * (uint32_t)KB * 512 + (lane & 31) * 16;
     s_dst = lds0 + kTBase + grp * 2 * kTSlot + GR * 128;   // + slot * kTSlot
   } else {
@@ -1008,7 +1013,7 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int M,
   wait_vmcnt<0>();
   if (grp == 0) block_barrier();
   block_barrier();
-  if constexpr (FUSE) tile_epilogue_mxq<BM, MTW, NTW, 4>(g, acc, e, M, m0, n0, row_base, mw, wj, lane, lds);
+  if constexpr (FUSE) tile_epilogue_mxq<BM, MTW, NTW, 4>(g, acc, ebso, M, m0, n0, row_base, mw, wj, lane, lds);
   else tile_epilogue<BM, MTW, NTW, 4, false>(g, acc, M, m0, n0, row_base, mw, nw, wj, lane, wave_active, lds);
 }
 
@@ -1101,7 +1106,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   const int hblocks = ws[kWsHeavyBlocks];
   const int ltotal = ws[kWsLightTotal], lsplit = ws[kWsLightSplit];
 #define ESMOE_CASE(MT_) \
-  case (MT_): gemm_tile<MT_, MX, FUSE>(g, e, M, t.m0, t.n0, lds); break;
+  case (MT_): gemm_tile<MT_, MX, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
 
   // Workgroup i runs on XCD i % 8 (HW_REG_XCC_ID = 20, bits [3:0], says so directly).  Of every 32 workgroups
   // of an XCD the last `light_share` start on the light items, the others on the heavy tickets; either kind
@@ -1172,8 +1177,13 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
       const int mid = (lo + hi) >> 1;
       if (sload(ws, (ws_rec(mid) + kind) * 4) <= idx) lo = mid; else hi = mid;
     }
-    const int first = sload(ws, (ws_rec(lo) + kind) * 4);
-    const int e = sload(ws, (ws_rec(lo) + kRecExpert) * 4), M = sload(ws, (ws_rec(lo) + kRecRows) * 4);
+    // the whole record in one load, then the expert's first row (and first scale row) through the scalar cache as
+    // well: a vector load here waits its turn behind the weight streams of the whole chip
+    const v4i rec = sload4(ws, ws_rec(lo) * 4);
+    const int first = __builtin_amdgcn_readfirstlane(light ? rec[kRecItem] : rec[kRecBlock]);
+    const int e = __builtin_amdgcn_readfirstlane(rec[kRecExpert]), M = __builtin_amdgcn_readfirstlane(rec[kRecRows]);
+    const int erow = sload(g.expert_offsets, e * 4);
+    const int ebso = MX ? sload(g.blockscale_offsets, e * 4) : 0;
     const int local = idx - first;
     TileCoord t;
     if (light) t = sched_decode_light(local, M, g.policy, half);
@@ -1200,19 +1210,19 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     bool hand_scheduled = false;
     if constexpr (MX) {
       if ((ESMOE_PPX_HEIGHTS & 2) && t.mt == 12) {
-        gemm_tile_pp_mx<12, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        gemm_tile_pp_mx<12, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
         hand_scheduled = true;
       } else if ((ESMOE_PPX_HEIGHTS & 1) && t.mt == 8) {
-        gemm_tile_pp_mx<8, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        gemm_tile_pp_mx<8, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
         hand_scheduled = true;
       }
     }
     if constexpr (!MX) {
       if ((ESMOE_PP_HEIGHTS & 2) && t.mt == 12) {
-        gemm_tile_pp<12, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        gemm_tile_pp<12, FUSE>(g, e, erow, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
         hand_scheduled = true;
       } else if ((ESMOE_PP_HEIGHTS & 1) && t.mt == 8) {
-        gemm_tile_pp<8, FUSE>(g, e, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
+        gemm_tile_pp<8, FUSE>(g, e, erow, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
         hand_scheduled = true;
       }
     }
@@ -1220,9 +1230,9 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
       if (!FUSE && t.nt == 2) {
         if constexpr (!FUSE) {
           switch (t.mt) {
-            case 1: gemm_tile<1, MX, false, 128>(g, e, M, t.m0, t.n0, lds); break;
-            case 2: gemm_tile<2, MX, false, 128>(g, e, M, t.m0, t.n0, lds); break;
-            case 4: gemm_tile<4, MX, false, 128>(g, e, M, t.m0, t.n0, lds); break;
+            case 1: gemm_tile<1, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
+            case 2: gemm_tile<2, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
+            case 4: gemm_tile<4, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
             default: break;
           }
         }
