@@ -244,6 +244,34 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, Acc& acc, int M
     return;
   }
   // epilogue: lane holds columns n0 + nw + nt*16 + 4*gq + [0,4) of token row m0 + mw + mt*16 + r
+  if constexpr (kWavesN == 4 && NTW == 4 && MTW >= 4) {
+    // Tall tiles: a wavefront holds 64 columns of its rows, 128 bytes of output per row.  Stored straight from the MFMA
+    // layout a store instruction writes 32-byte pieces of sixteen rows; passed through LDS (the ring is free, and each
+    // wavefront reads back only what it wrote itself, so no barrier) it writes whole 128-byte lines of eight rows, in half
+    // as many instructions.  Rows are 144 bytes apart in LDS to spread the banks.
+    constexpr int kRows = MTW * 16, kStride = 144;
+    uint8_t* const region = lds + ((mw / kRows) * kWavesN + wn) * (kRows * kStride);
+#pragma unroll
+    for (int mt = 0; mt < MTW; mt++) {
+#pragma unroll
+      for (int nt = 0; nt < NTW; nt++) {
+        const v4f v = {acc[nt][mt][0], acc[nt][mt][1], acc[nt][mt][2], acc[nt][mt][3]};
+        uint8_t* const dst = region + (mt * 16 + r) * kStride + nt * 32 + gq * 8;
+        if (g.out_dtype == 0) *(bf16x4*)dst = __builtin_convertvector(v, bf16x4);
+        else *(f16x4*)dst = __builtin_convertvector(v, f16x4);
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int rr = lane >> 3, ch = lane & 7;
+#pragma unroll
+    for (int i = 0; i < kRows / 8; i++) {
+      const int row = i * 8 + rr;
+      const int m = m0 + mw + row;
+      const v4i line = *(const v4i*)(region + row * kStride + ch * 16);
+      if (wave_active && m < M) *(v4i*)((uint8_t*)g.out + ((row_base + m) * (long)N + n0 + nw) * 2 + ch * 16) = line;
+    }
+    return;
+  }
   if (wave_active) {
 #pragma unroll
     for (int mt = 0; mt < MTW; mt++) {
