@@ -172,6 +172,19 @@ struct TileGeom {
   static_assert(kNBuf >= 2, "ring too small");
 };
 
+// The fused epilogues gather a tile's quantised bytes in LDS, BM rows of 128 bytes `stride` apart, and the workgroup
+// writes them from there: eight lanes a row, a whole 128-byte line per row where the MFMA layout would give 16-byte
+// pieces.  `dst` is the tile's first byte of the expert's row 0 (row pitch `pitch`); rows at or past M are not written.
+template <int BM>
+__device__ __forceinline__ void store_staged_rows(const uint8_t* stage, int stride, uint8_t* dst, int pitch, int M, int m0) {
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int row = tid >> 3; row < BM; row += kThreads / 8) {
+    const int m = m0 + row;
+    if (m < M) *(v4i*)(dst + (long)m * pitch + (tid & 7) * 16) = *(const v4i*)(stage + row * stride + (tid & 7) * 16);
+  }
+}
+
 // Epilogue of a tile: `acc[nt][mt][i]` holds, for this lane, columns n0 + nw + nt*16 + 4*gq + i of token row
 // m0 + mw + mt*16 + r (gq = lane / 16, r = lane % 16).  Plain form: convert and store.  FUSE: SwiGLU and the 1x128
 // quantisation (the wavefront's first NTW/2 column tiles are gate columns, the rest the matching up columns).
@@ -187,6 +200,8 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, Acc& acc, int M
     // sequence: projection rounded to the output type, silu(gate) * up in fp32, rounded to the output type, then
     // the 1x128 quantisation (block maximum floored at 1e-4, multiplier (1/amax)*448, scale amax*(1/448)).
     constexpr int kHalf = NTW / 2, kRW = NTW * 16;
+    constexpr int kStageOff = 4096, kStageStride = 144;   // behind s_amax: BM rows of the tile's 128 output bytes
+    static_assert(kWavesN * BM * 4 <= kStageOff, "s_amax and the stage overlap");
     const bool f16 = g.out_dtype != 0;
     float* s_amax = (float*)lds;   // [kWavesN][BM]; the ring is free: every wavefront has left the K loop
     float h[MTW][kHalf][4];
@@ -226,21 +241,22 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, Acc& acc, int M
       amax = __builtin_fmaxf(amax, 1e-4f);
       const float mult = (1.0f / amax) * 448.0f;
       const int m = m0 + row;
-      if (m < M) {
-        uint8_t* qrow = (uint8_t*)g.q_out + (row_base + m) * (long)inter + (n0 >> 1) + wn * (kRW / 2) + gq * 4;
+      // the row's 128 quantised bytes are gathered in LDS (a lane holds 4 of them per column tile) and leave as one line
+      uint8_t* const qstage = lds + kStageOff + row * kStageStride + wn * (kRW / 2) + gq * 4;
 #pragma unroll
-        for (int nt = 0; nt < kHalf; nt++) {
-          float y[4];
+      for (int nt = 0; nt < kHalf; nt++) {
+        float y[4];
 #pragma unroll
-          for (int i = 0; i < 4; i++) y[i] = __builtin_amdgcn_fmed3f(h[mt][nt][i] * mult, -448.f, 448.f);
-          int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
-          w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
-          *(int*)(qrow + nt * 16) = w0;
-        }
-        if (gq == 0 && wn == 0) g.scales_out[(row_base + m) * (long)(inter >> 7) + (n0 >> 8)] = amax * (1.0f / 448.0f);
+        for (int i = 0; i < 4; i++) y[i] = __builtin_amdgcn_fmed3f(h[mt][nt][i] * mult, -448.f, 448.f);
+        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+        *(int*)(qstage + nt * 16) = w0;
       }
+      if (m < M && gq == 0 && wn == 0) g.scales_out[(row_base + m) * (long)(inter >> 7) + (n0 >> 8)] = amax * (1.0f / 448.0f);
     }
-    __syncthreads();   // s_amax is ring memory: the next tile's copies must not land before every lane has read it
+    __syncthreads();
+    store_staged_rows<BM>(lds + kStageOff, kStageStride, (uint8_t*)g.q_out + row_base * (long)inter + (n0 >> 1), inter, M, m0);
+    __syncthreads();   // the stage and s_amax are ring memory: the next tile's copies must not land before they are read
     return;
   }
   // epilogue: lane holds columns n0 + nw + nt*16 + 4*gq + [0,4) of token row m0 + mw + mt*16 + r
@@ -310,6 +326,8 @@ __device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, i
   const int r = lane & 15, gq = lane >> 4;
   const bool f16 = g.out_dtype != 0;
   const int inter = g.n >> 1;
+  constexpr int kCodeOff = 4096, kStageOff = 5120, kStageStride = 144;   // behind s_amax: scale dwords, then the byte rows
+  static_assert(kWavesN * BM * 4 <= kCodeOff && BM * 4 <= kStageOff - kCodeOff, "s_amax, the scale dwords and the stage overlap");
   float* s_amax = (float*)lds;   // [kWavesN][BM]; the ring is free: every wavefront has left the K loop
   float h[MTW][kHalf][4], amaxv[MTW];
 #pragma unroll
@@ -350,22 +368,26 @@ __device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, i
     if constexpr (kPair) amax = __builtin_fmaxf(amax, s_amax[(wn ^ 1) * BM + row]);
     const int code = mx_scale_code(amax);
     const float inv = mx_scale_inverse(amax, code);
-    if (m < M) {
-      uint8_t* qrow = (uint8_t*)g.q_out + (row_base + m) * (long)inter + (n0 >> 1) + wn * (kRW / 2) + gq * 4;
+    // the row's 128 quantised bytes and its four scale bytes (one dword of the swizzled scale tile) are gathered in LDS
+    uint8_t* const qstage = lds + kStageOff + row * kStageStride + wn * (kRW / 2) + gq * 4;
 #pragma unroll
-      for (int nt = 0; nt < kHalf; nt++) {
-        float y[4];
+    for (int nt = 0; nt < kHalf; nt++) {
+      float y[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) y[i] = __builtin_amdgcn_fmed3f(h[mt][nt][i] * inv, -448.f, 448.f);
-        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
-        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
-        *(int*)(qrow + nt * 16) = w0;
-      }
+      for (int i = 0; i < 4; i++) y[i] = __builtin_amdgcn_fmed3f(h[mt][nt][i] * inv, -448.f, 448.f);
+      int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
+      w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+      *(int*)(qstage + nt * 16) = w0;
     }
-    if (gq == 0 && (!kPair || (wn & 1) == 0) && m < m_pad) {
-      sf_e[((long)(m >> 7) * (inter >> 7) + (cblk >> 2)) * 512 + (m & 31) * 16 + ((m & 127) >> 5) * 4 + (cblk & 3)] =
-          (uint8_t)(m < M ? code : 0);
-    }
+    if (gq == 0 && (!kPair || (wn & 1) == 0)) lds[kCodeOff + row * 4 + (cblk & 3)] = (uint8_t)(m < M ? code : 0);
+  }
+  __syncthreads();
+  store_staged_rows<BM>(lds + kStageOff, kStageStride, (uint8_t*)g.q_out + row_base * (long)inter + (n0 >> 1), inter, M, m0);
+  for (int row = threadIdx.x; row < BM; row += kThreads) {
+    const int m = m0 + row;
+    if (m < m_pad)
+      *(uint32_t*)(sf_e + ((long)(m >> 7) * (inter >> 7) + (n0 >> 8)) * 512 + (m & 31) * 16 + ((m & 127) >> 5) * 4) =
+          *(const uint32_t*)(lds + kCodeOff + row * 4);
   }
   // rows of the expert's last scale tile that lie below this tile: the tile's four scale columns are one dword
   if (m0 + BM >= M) {
@@ -373,7 +395,7 @@ __device__ __forceinline__ void tile_epilogue_mxq(const GemmArgs& g, Acc& acc, i
       *(uint32_t*)(sf_e + ((long)(m >> 7) * (inter >> 7) + (n0 >> 8)) * 512 + (m & 31) * 16 + ((m & 127) >> 5) * 4) = 0u;
     }
   }
-  if constexpr (kPair) __syncthreads();   // s_amax is ring memory: the next tile's copies must not land before it is read
+  __syncthreads();   // the stages (and s_amax) are ring memory: the next tile's copies must not land before they are read
 }
 
 // FUSE: the weights are a gate_up projection [E, 2I, K] (gate rows first) and the tile's 256 weight rows are 128 gate
