@@ -227,7 +227,7 @@ def emit(name, mtw, fuse):
 # rows behind a weight stage, 2 for the group's token rows behind its token stage); every wavefront issues one
 # 1 KB scale copy per K block so that the counted waits are the same for all (wavefront 0: weight scales of K block
 # kb + 2, wavefronts 1 and 5: their group's token scales of kb + 1, the others re-read one line into a spare area).
-# A lane reads the scale dword of its row and shifts its K sub-block's byte (lane / 16) down to byte 0.
+# A lane reads, of the scale dword of its row, the byte of its K sub-block (lane / 16).
 class MxPlan:
     def __init__(self, mtw, fuse=False):
         self.mtw = mtw
@@ -270,17 +270,15 @@ def mx_memory_phase(p):
                 L.append(f"ds_read_b128 {d}, %[{a}]" + (f" offset:{off}" if off else ""))
     for d, a, off in rd:
         L.append(f"ds_read_b128 {d}, %[{a}]" + (f" offset:{off}" if off else ""))
+    # a lane reads the one scale byte it feeds (its addresses point at byte lane / 16 of the row's scale dword): the
+    # MFMA takes byte 0 of the register, and nothing stands between the LDS wait and the barrier
     for nt in range(4):
         # plain: n-tiles 2, 3 are the next 32-row quarter of the same scale tile; gate_up: the second tile (up rows)
         off = (nt & 1) * 256 + (nt >> 1) * (512 if p.fuse else 4)
-        L.append(f"ds_read_b32 v{p.sfw + nt}, %[sfwl]" + (f" offset:{off}" if off else ""))
+        L.append(f"ds_read_u8 v{p.sfw + nt}, %[sfwl]" + (f" offset:{off}" if off else ""))
     for mt in range(p.mtw):
-        L.append(f"ds_read_b32 v{p.sfa + mt}, %[sfa{mt}]")
+        L.append(f"ds_read_u8 v{p.sfa + mt}, %[sfa{mt}]")
     L.append("s_waitcnt lgkmcnt(0)")
-    for nt in range(4):
-        L.append(f"v_lshrrev_b32 v{p.sfw + nt}, %[sh], v{p.sfw + nt}")
-    for mt in range(p.mtw):
-        L.append(f"v_lshrrev_b32 v{p.sfa + mt}, %[sh], v{p.sfa + mt}")
     L.append(f"s_waitcnt vmcnt({p.ntc + 5}) ; explicit")
     L.append("s_barrier")
     return L
@@ -354,7 +352,7 @@ def emit_mx(name, mtw, fuse=False):
     outs += [f'[sfa{mt}] "+v"(sfal[{mt}])' for mt in range(mtw)]
     outs += ['[la] "+s"(la)', '[lw] "+s"(lw)', '[ls] "+s"(ls)', '[td] "+s"(td)', '[woff] "+s"(woff)', '[rem] "+s"(rem)']
     print(f"#define {name}_OUTS " + ", ".join(outs))
-    ins = ['[wfrag] "v"(wfrag)', '[sfwrd] "v"(sfw_rd)', '[sh] "v"(shift)', '[ap] "s"(a_ptr)', '[wp] "s"(w_ptr)', '[sp] "s"(s_ptr)',
+    ins = ['[wfrag] "v"(wfrag)', '[sfwrd] "v"(sfw_rd)', '[ap] "s"(a_ptr)', '[wp] "s"(w_ptr)', '[sp] "s"(s_ptr)',
            '[lwbase] "s"(lwbase)', '[lwend] "s"(lwend)', '[lsinc] "s"(lsinc)', '[lsend] "s"(lsend)', '[lswrap] "s"(lswrap)',
            '[sthr] "s"(sthr)']
     print(f"#define {name}_INS " + ", ".join(ins))

@@ -990,15 +990,15 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int er
   // weight scale dword of row nw + nt*16 + r: n-tile nt at + (nt & 1)*256 + (nt >> 1)*4.  FUSE: the wavefront's gate
   // rows are rows wj*32 + nt*16 + r of the first tile (n-tiles 0, 1), its up rows the same rows of the second (2, 3):
   // n-tile nt at + (nt & 1)*256 + (nt >> 1)*512
-  const uint32_t sfw_rd = FUSE ? lds0 + kBN * 128 + r * 16 + wj * 4
-                               : lds0 + kBN * 128 + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16;
+  // (+ gq: of a row's scale dword a lane reads the byte of its own K sub-block)
+  const uint32_t sfw_rd = (FUSE ? lds0 + kBN * 128 + r * 16 + wj * 4
+                                : lds0 + kBN * 128 + (nw >> 7) * 512 + ((nw & 127) >> 5) * 4 + ((nw & 31) + r) * 16) + gq;
   uint32_t sfa_rd[MTW];
 #pragma unroll
   for (int mt = 0; mt < MTW; mt++) {
     const int ml = ((m0 + mw) & 127) + mt * 16 + r;   // row inside the group's two scale tiles
-    sfa_rd[mt] = lds0 + kTBase + grp * 2 * kTSlot + GR * 128 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4;
+    sfa_rd[mt] = lds0 + kTBase + grp * 2 * kTSlot + GR * 128 + (ml >> 7) * 512 + (ml & 31) * 16 + ((ml & 127) >> 5) * 4 + gq;
   }
-  const uint32_t shift = gq * 8;
 
   v4f acc[NTW][MTW];
 #pragma unroll
