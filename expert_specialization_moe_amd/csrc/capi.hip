@@ -157,7 +157,8 @@ int check_common(const void* out, const void* a, const void* b, const int32_t* p
   if (!workspace || workspace_bytes < esmoe_gemm_workspace_bytes(num_experts))
     return fail(ESMOE_ERR_WORKSPACE_TOO_SMALL, "workspace of %zu bytes is smaller than the %zu required",
                 workspace_bytes, esmoe_gemm_workspace_bytes(num_experts));
-  if ((uintptr_t)workspace % 4) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace must be 4-byte aligned");
+  // (the kernel reads a schedule record with one 16-byte scalar load)
+  if ((uintptr_t)workspace % 16) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
   if ((uintptr_t)a % 16 || (uintptr_t)b % 16 || (uintptr_t)out % 8)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "a and b must be 16-byte aligned, out 8-byte aligned");
   return 0;

@@ -36,7 +36,8 @@ extern "C" {
 #define ESMOE_MAX_EXPERTS 1024 /* same limit as the reference, es_fp8_blockwise_launcher.cuh:53 */
 
 /* Bytes of device scratch the two GEMM entry points need for `num_experts` experts
- * (the device-built tile schedule and its work counter). */
+ * (the device-built tile schedule and its work counter).  The scratch must be 16-byte aligned (device allocations are);
+ * its contents before a call do not matter. */
 size_t esmoe_gemm_workspace_bytes(int num_experts);
 
 /*
