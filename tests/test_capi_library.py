@@ -38,6 +38,11 @@ def test_argument_validation_needs_no_gpu(esmoe):
     assert rc == -1 and "force_bm" in _native.last_error()
     rc = lib.esmoe_fp8_blockwise_grouped_mm(p, 0, p, p, p, p, p, p, 4, 10, 128, 128, 0, p, 8, None)
     assert rc == -2 and "workspace" in _native.last_error()
+    # a workspace that is not 16-byte aligned (the kernel reads its schedule records with 16-byte scalar loads)
+    base = ctypes.addressof(buf)
+    odd = ctypes.c_void_p(base + (16 - base % 16) % 16 + 4)
+    rc = lib.esmoe_fp8_blockwise_grouped_mm(p, 0, p, p, p, p, p, p, 4, 10, 128, 128, 0, odd, 2048, None)
+    assert rc == -1 and "16-byte aligned" in _native.last_error()
     rc = lib.esmoe_mxfp8_grouped_quant(p, 7, p, p, p, p, p, 4, 10, 128, 128, None)
     assert rc == -1 and "in_dtype" in _native.last_error()
     rc = lib.esmoe_mxfp8_grouped_quant(p, 0, p, p, p, p, p, 4, 10, 100, 128, None)
