@@ -1,11 +1,15 @@
-"""The K loops of the grouped GEMM must contain no memory wait that the compiler added on its own.
+"""Properties of the compiled grouped GEMM kernels that no result shows and every timing does.
+
+1. The K loops must contain no memory wait that the compiler added on its own.
 
 The loops keep several K blocks of asynchronous global->LDS copies in flight and wait for them with explicit
 `s_waitcnt vmcnt(N)` instructions (inline assembly, tagged "explicit").  The compiler counts only the loads and
 stores it emitted itself; when it believes one of those is still outstanding on entry to a K loop it puts a
 `s_waitcnt vmcnt(small)` of its own into the loop, which in reality also waits for nearly all copies in flight and
-costs 30-40 % of the loop's speed with no wrong result to give it away.  This test compiles the kernel to assembly
+costs 30-40 % of the loop's speed with no wrong result to give it away.  The test compiles the kernel to assembly
 (no GPU needed) and checks every loop that contains MFMAs.
+
+2. The kernels must not spill a vector register (test_grouped_gemm_kernels_spill_no_vector_register).
 """
 import importlib.util
 import os
@@ -53,14 +57,30 @@ def _mfma_loops(asm_text):
     return {k: b for k, b in blocks.items() if k[2] >= 2 and any("v_mfma" in t for _, t in b)}
 
 
-def test_no_compiler_inserted_vmcnt_wait_in_k_loops(tmp_path):
+@pytest.fixture(scope="module")
+def kernel_asm(tmp_path_factory):
     build = _build_module()
     if not (os.path.exists(build.HIPCC) or shutil.which(build.HIPCC)):
         pytest.skip("hipcc not available")
-    out = tmp_path / "grouped_gemm.s"
+    out = tmp_path_factory.mktemp("asm") / "grouped_gemm.s"
     cmd = [build.HIPCC] + build.HIP_FLAGS + ["--cuda-device-only", "-S", os.path.join(build.CSRC, "grouped_gemm.hip"), "-o", str(out)]
     subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-    loops = _mfma_loops(out.read_text())
+    return out.read_text()
+
+
+def test_grouped_gemm_kernels_spill_no_vector_register(kernel_asm):
+    """The four grouped GEMM kernels use every vector register there is (two wavefronts of 256 per SIMD) and must not
+    spill one: a spill makes the launch set up scratch memory and puts the compiler's own full memory waits around the
+    reloads.  The code object's metadata says how many were spilled and how much scratch a lane gets."""
+    kernels = re.findall(r"\.name:\s+(_ZN5esmoe19grouped_gemm_kernel\w+)\n\s+\.private_segment_fixed_size:\s+(\d+)\n(?:.*\n)*?\s+\.vgpr_spill_count:\s+(\d+)",
+                         kernel_asm)
+    assert len(kernels) == 4, kernels
+    for name, scratch, spilled in kernels:
+        assert int(scratch) == 0 and int(spilled) == 0, (name, scratch, spilled)
+
+
+def test_no_compiler_inserted_vmcnt_wait_in_k_loops(kernel_asm):
+    loops = _mfma_loops(kernel_asm)
     # 6 tile heights x {fp8-blockwise, mxfp8}
     assert len(loops) >= 12, sorted(loops)
     stray = [(k, n, t) for k, b in loops.items() for n, t in b if "s_waitcnt" in t and "vmcnt" in t and "explicit" not in t]
