@@ -57,7 +57,8 @@ def parse():
     ap.add_argument("--settle-ms", type=float, default=200.0,
                     help="untimed: run the step for this many milliseconds before the warm-up steps, so that a small "
                          "--warmup does not time the chip's clock ramp (0 = off)")
-    ap.add_argument("--config", default="c1", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--config", default="c1", choices=["c1", "c2", "c3", "c4", "dense", "dense_mx"],
+                    help="dense, dense_mx: one expert of 12288 rows, N=4096, K=7168 (fp8-blockwise, mxfp8): the tall tiles alone")
     ap.add_argument("--tokens", type=int, default=8192, help="c3 only")
     ap.add_argument("--routing", default="zipf", choices=["zipf", "uniform"], help="c3 only")
     ap.add_argument("--seed", type=int, default=0)

@@ -66,7 +66,7 @@ class Problem:
 
 
 def config_problem(name, seed=0, tokens=None, routing="zipf"):
-    """The benchmark configurations by name: c0 .. c4."""
+    """The benchmark configurations by name: c0 .. c4, and a single large expert (dense, dense_mx)."""
     if name == "c0":
         rng = np.random.default_rng(seed)
         return Problem("c0", 256, 512, [int(v) for v in rng.integers(1, 65, size=8)])
@@ -82,6 +82,10 @@ def config_problem(name, seed=0, tokens=None, routing="zipf"):
     if name == "c4":
         return Problem("c4", 4096, 7168, zipf_multinomial_rows(seed, 8192, 32, 1.0), kind="mxfp8",
                        meta={"rows": 8192, "zipf_s": 1.0})
+    if name in ("dense", "dense_mx"):
+        # one large expert: what the tall tiles do when nothing else runs beside them (no counterpart among the
+        # reference's benchmark shapes; it isolates the matrix-bound part of c1/c3/c4)
+        return Problem(name, 4096, 7168, [12288], kind="mxfp8" if name == "dense_mx" else "fp8_blockwise", meta={"rows": 12288})
     raise ValueError(name)
 
 
