@@ -41,7 +41,7 @@ a write of m0 from the copy that uses it.
 import sys
 
 NT = 4
-ABLATE = set()   # timing experiments only (results wrong): "fma", "copy", "roll", "read", "scread", "barrier", "vmwait";
+ABLATE = set()   # timing experiments only (results wrong): "fma", "copy" ("copyw", "copyt", "copys": weight, token, scale copies only), "roll", "read", "scread", "barrier", "vmwait";
                  # "bookodd": bookkeeping behind every second MFMA instead (results right);
                  # "prioN" / "mprioN": the matrix / memory phase at wave priority N ("prio0": none; results right);
                  # "latebar": every LDS read of the memory phase waited for in front of its barrier (results right)
@@ -231,6 +231,9 @@ def ablated(lines):
         if "halffma" in ABLATE and l.startswith("v_fmac") and l.split("]")[0][-1] in "13":
             continue
         if "copy" in ABLATE and l.startswith("global_load_lds"):
+            continue
+        if any(w in ABLATE and l.startswith("global_load_lds") and f"%[{op}" in l
+               for w, op in (("copyw", "vw"), ("copyt", "va"), ("copys", "vs]"))):
             continue
         if "read" in ABLATE and l.startswith("ds_read_b128") and "%[w" in l:
             continue
