@@ -181,7 +181,7 @@ __device__ __forceinline__ void store_staged_rows(const uint8_t* stage, int stri
 #pragma unroll
   for (int row = tid >> 3; row < BM; row += kThreads / 8) {
     const int m = m0 + row;
-    if (m < M) *(v4i*)(dst + (long)m * pitch + (tid & 7) * 16) = *(const v4i*)(stage + row * stride + (tid & 7) * 16);
+    if (m < M) __builtin_nontemporal_store(*(const v4i*)(stage + row * stride + (tid & 7) * 16), (v4i*)(dst + (long)m * pitch + (tid & 7) * 16));
   }
 }
 
@@ -264,7 +264,9 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, Acc& acc, int M
     // Tall tiles: a wavefront holds 64 columns of its rows, 128 bytes of output per row.  Stored straight from the MFMA
     // layout a store instruction writes 32-byte pieces of sixteen rows; passed through LDS (the ring is free, and each
     // wavefront reads back only what it wrote itself, so no barrier) it writes whole 128-byte lines of eight rows, in half
-    // as many instructions.  Rows are 144 bytes apart in LDS to spread the banks.
+    // as many instructions.  Rows are 144 bytes apart in LDS to spread the banks.  Whole lines of output are stored with the
+    // non-temporal hint: nothing in this launch reads them, and they should not push operand panels out of L2 (C4 -3 %,
+    // C1 -1.8 %; the short tiles' 8-byte pieces are better off merging in L2: C2 +0.6 % with the hint).
     constexpr int kRows = MTW * 16, kStride = 144;
     uint8_t* const region = lds + ((mw / kRows) * kWavesN + wn) * (kRows * kStride);
 #pragma unroll
@@ -284,7 +286,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& g, Acc& acc, int M
       const int row = i * 8 + rr;
       const int m = m0 + mw + row;
       const v4i line = *(const v4i*)(region + row * kStride + ch * 16);
-      if (wave_active && m < M) *(v4i*)((uint8_t*)g.out + ((row_base + m) * (long)N + n0 + nw) * 2 + ch * 16) = line;
+      if (wave_active && m < M) __builtin_nontemporal_store(line, (v4i*)((uint8_t*)g.out + ((row_base + m) * (long)N + n0 + nw) * 2 + ch * 16));
     }
     return;
   }
