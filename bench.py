@@ -20,9 +20,9 @@ import torch
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "gemm"): 1.558e9,     # FETCH 734,317.9 x 2.000 KiB + WRITE 52,690.0 x 1.000 KiB
-    ("c2", "gemm"): 4.485e8,     # FETCH 217,193.9 x 2.000 KiB + WRITE 3,630.6 x 1.000 KiB
-    ("c4", "gemm"): 1.458e9,     # FETCH 679,152.4 x 2.000 KiB + WRITE 65,594.3 x 1.000 KiB
+    ("c1", "gemm"): 1.546e9,     # FETCH 728,712.7 x 2.000 KiB + WRITE 52,745.4 x 1.000 KiB
+    ("c2", "gemm"): 4.486e8,     # FETCH 217,244.4 x 2.000 KiB + WRITE 3,630.7 x 1.000 KiB
+    ("c4", "gemm"): 1.455e9,     # FETCH 677,660.2 x 2.000 KiB + WRITE 65,715.8 x 1.000 KiB
     ("c4", "quant"): 1.786e8,    # FETCH 57,399.0 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
 }
 
