@@ -94,3 +94,21 @@ def test_reads_left_out_at_the_first_barrier_are_the_groups_own(name, lines):
             assert outstanding, f"{name}: nothing is left out at the barrier (the wait in front of it is the old, full one)"
             assert all(any(o in l for o in own) for l in outstanding), f"{name}: {outstanding}"
             break
+
+
+def test_every_statement_raises_the_priority_for_its_matrix_phase_only():
+    """The generated header: one `s_setprio 3` right after the barrier that ends the memory phase (and the wait for the
+    group's own reads), one `s_setprio 0` in front of the wait and barrier that end the matrix phase, so that the
+    wavefront leaves every statement, and with it the K loop, at priority 0."""
+    text = open(os.path.join(ROOT, "expert_specialization_moe_amd", "csrc", "pp_phase.h")).read()
+    bodies = re.findall(r"#define (\w+_BODY\w*) \\\n((?:  \".*\n)+)", text)
+    assert len(bodies) == 16
+    for name, body in bodies:
+        lines = [l.strip().strip("\\").strip().strip('"').replace("\\n\\t", "") for l in body.splitlines()]
+        prio = [(i, l) for i, l in enumerate(lines) if l.startswith("s_setprio")]
+        barriers = [i for i, l in enumerate(lines) if l == "s_barrier"]
+        mfma = [i for i, l in enumerate(lines) if l.startswith("v_mfma")]
+        assert [l for _, l in prio] == ["s_setprio 3", "s_setprio 0"], name
+        assert len(barriers) == 2, name
+        assert barriers[0] < prio[0][0] < mfma[0], name
+        assert mfma[-1] < prio[1][0] < barriers[1], name
