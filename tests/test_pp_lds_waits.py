@@ -112,3 +112,11 @@ def test_every_statement_raises_the_priority_for_its_matrix_phase_only():
         assert len(barriers) == 2, name
         assert barriers[0] < prio[0][0] < mfma[0], name
         assert mfma[-1] < prio[1][0] < barriers[1], name
+
+
+def test_committed_header_is_what_the_generator_writes():
+    import subprocess
+    import sys
+    csrc = os.path.join(ROOT, "expert_specialization_moe_amd", "csrc")
+    out = subprocess.run([sys.executable, os.path.join(csrc, "gen_pp_phase.py")], capture_output=True, text=True, check=True).stdout
+    assert out == open(os.path.join(csrc, "pp_phase.h")).read(), "pp_phase.h is stale: python gen_pp_phase.py > pp_phase.h"
