@@ -26,4 +26,7 @@ Parity status per function (what pins it is in ``tests/test_oracle_*.py``):
 * ``mxfp8.sf_offset``  pinned: literal enumeration of the CuTe layout
   ``((32,4),4):((16,4),1)`` tiled K-fastest.
 * ``mxfp8.grouped_mm``  pinned: same exact-case set as ``fp8_blockwise.grouped_mm``.
+* ``torch_path.scaled_mm / mx_scaled_mm``  (the benchmark's CPU baseline: the reference's
+  torch path in stock torch ops)  pinned: against the two ``grouped_mm`` above and an
+  exact small-integer case.
 """

@@ -38,9 +38,11 @@ def check_close(y, ref, what=""):
 
 
 def check_ulps(y, ref, out_dtype, what="", ulps=2.0, abs_rms=2e-3):
-    """Tight form for a kernel whose accumulation order the oracle follows: every element within `ulps` units in
-    the last place of the output type (bf16: 2^-8 relative, fp16: 2^-11) plus abs_rms of the result's rms, which
-    covers cancellation between K blocks (fp32 sums taken in another order inside a block)."""
+    """Tight form of the tolerance: every element within `ulps` units in the last place of the output type (bf16:
+    2^-8 relative, fp16: 2^-11) plus abs_rms of the result's rms.  The oracle dequantises and then multiplies in
+    fp32, the kernels scale per K block (fp8-blockwise) or inside the MFMA (mxfp8) and sum in another order: both
+    are fp32 evaluations of the same real number, and the rms term is what absorbs their difference where K blocks
+    cancel."""
     y = np.asarray(y, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     ok = np.isfinite(ref)

@@ -38,7 +38,7 @@ def test_c0_through_torch_op(esmoe):
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
 def test_forced_tile_shapes(esmoe, force_bm, out_dtype):
     """Every tile height of the menu and the device schedule (0), both output types, against the oracle; also the
-    tight form of the tolerance (the oracle accumulates per K block in the kernel's order)."""
+    tight form of the tolerance (helpers.check_ulps)."""
     from expert_specialization_moe_amd import _native
     from expert_specialization_moe_amd import workloads as W
 
@@ -52,11 +52,12 @@ def test_forced_tile_shapes(esmoe, force_bm, out_dtype):
     H.check_ulps(y, ref, out_dtype, f"ragged bm={force_bm}")
 
 
-@pytest.mark.parametrize("k", [512, 1024, 1536])
+@pytest.mark.parametrize("k", [128, 384, 512, 640, 1024, 1536])
 @pytest.mark.parametrize("force_bm", [0, 128, 192])
-def test_tall_tiles_with_k_a_multiple_of_512(esmoe, force_bm, k):
-    """K % 512 == 0 selects the hand-scheduled K block of the 192-row (and, when enabled, 128-row) tiles: one to three
-    scale chunks, full and ragged tiles, a last column tile that is half empty, against the oracle."""
+def test_tall_tiles_with_whole_and_ragged_scale_chunks(esmoe, force_bm, k):
+    """The hand-scheduled K block of the 128- and 192-row tiles fetches the activation scales four K blocks at a time:
+    K of one, three and five K blocks (a single short chunk; a last chunk that overlaps the one before) and of one to
+    three whole chunks, full and ragged tiles, a last column tile that is half empty, against the oracle."""
     from expert_specialization_moe_amd import _native
     from expert_specialization_moe_amd import workloads as W
 

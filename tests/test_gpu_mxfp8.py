@@ -70,6 +70,70 @@ def test_mx_gemm_parity(esmoe, force_bm, out_dtype):
     assert np.isfinite(y).all()
 
 
+@pytest.mark.parametrize("force_bm", [0, 16, 32, 64, 128, 192])
+def test_mx_tiles_exact_with_distinct_scale_bytes(esmoe, force_bm):
+    """Small-integer e4m3 operands and E8M0 scale bytes that differ for every (token row, 32-wide K sub-block) and every
+    (weight row, K sub-block): every partial sum is exact in fp32, so the result must EQUAL the fp64 evaluation rounded
+    once, and a scale byte taken from a neighbouring row, sub-block, K block or scale tile shows as a wrong value, not as
+    rounding.  Experts of 200 / 385 / 530 rows make 192-row tiles start in the middle of a 128-row scale tile.  Every
+    tile height, and the fused SwiGLU + quantisation epilogue against the stand-alone quantiser fed the exact result."""
+    from expert_specialization_moe_amd import _native
+    from expert_specialization_moe_amd import workloads as W
+    from oracle import fp8
+
+    rows, n, k = [200, 0, 385, 33, 530], 512, 2048
+    kc = k // 32
+    rng = np.random.default_rng(12)
+    e, total = len(rows), sum(rows)
+    ai = rng.integers(-2, 3, size=(total, k)).astype(np.float32)
+    bi = rng.integers(-2, 3, size=(e, n, k)).astype(np.float32)
+    ca = rng.integers(125, 130, size=(total, kc)).astype(np.uint8)      # 2^-2 .. 2^2 per (row, sub-block)
+    cb = rng.integers(125, 130, size=(e, n, kc)).astype(np.uint8)
+    offs = W.offsets_of(rows)
+    bso_np, sf_rows = W.blockscale_offsets_of(rows)
+    sfa = np.zeros(sf_rows * kc, dtype=np.uint8)
+    for g, (m, off) in enumerate(zip(rows, offs)):
+        if m:
+            omx.swizzle_scales(ca[off:off + m], k, out=sfa, base=int(bso_np[g]) * kc)
+    sfb = np.zeros(e * n * kc, dtype=np.uint8)
+    for g in range(e):
+        omx.swizzle_scales(cb[g], k, out=sfb, base=g * n * kc)
+    ops = {
+        "a": torch.from_numpy(fp8.e4m3fn_encode_rne(ai)).cuda().view(torch.float8_e4m3fn),
+        "b_phys": torch.from_numpy(fp8.e4m3fn_encode_rne(bi)).cuda().view(torch.float8_e4m3fn),
+        "sfa": torch.from_numpy(sfa).cuda().view(sf_rows, kc), "sfb_phys": torch.from_numpy(sfb).cuda().view(e, n, kc),
+        "problem_sizes": torch.tensor([[m, n, k] for m in rows], dtype=torch.int32, device="cuda"),
+        "expert_offsets": torch.tensor(offs, dtype=torch.int32, device="cuda"),
+        "blockscale_offsets": torch.tensor(bso_np, dtype=torch.int32, device="cuda"),
+        "output": torch.full((total, n), float("nan"), dtype=torch.bfloat16, device="cuda"),
+    }
+    y = H.f32(H.capi_mx_mm(_native, ops, force_bm=force_bm))
+    want = np.empty((total, n), dtype=np.float32)
+    for g, (m, off) in enumerate(zip(rows, offs)):
+        if m:
+            da = ai[off:off + m].astype(np.float64) * np.repeat(np.exp2(ca[off:off + m].astype(np.float64) - 127), 32, 1)
+            db = bi[g].astype(np.float64) * np.repeat(np.exp2(cb[g].astype(np.float64) - 127), 32, 1)
+            want[off:off + m] = fp8.bf16_round((da @ db.T).astype(np.float32))
+            assert np.array_equal(y[off:off + m], want[off:off + m]), f"expert {g} ({m} rows), tile height {force_bm}"
+    # fused epilogue: the bytes and scale bytes of the stand-alone quantiser applied to the (exact) projection
+    inter = n // 2
+    lib = _native.lib
+    ws_bytes = lib.esmoe_gemm_workspace_bytes(e)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device="cuda")
+    q = torch.full((total, inter), 0x55, dtype=torch.uint8, device="cuda")
+    sf = torch.zeros((sf_rows, inter // 32), dtype=torch.uint8, device="cuda")
+    rc = lib.esmoe_mxfp8_grouped_mm_swiglu_quant(
+        H.ptr(q), H.ptr(sf), 0, H.ptr(ops["a"]), H.ptr(ops["b_phys"]), H.ptr(ops["sfa"]), H.ptr(ops["sfb_phys"]),
+        H.ptr(ops["problem_sizes"]), H.ptr(ops["expert_offsets"]), H.ptr(ops["blockscale_offsets"]), e, total, sf_rows, n, k,
+        force_bm, H.ptr(ws), ws_bytes, H.stream_ptr())
+    assert rc == 0, _native.last_error()
+    q2, sf2 = torch.zeros_like(q), torch.zeros_like(sf)
+    esmoe.es_swiglu_mxfp8_grouped_quant(torch.from_numpy(want).cuda().to(torch.bfloat16), ops["problem_sizes"], ops["expert_offsets"],
+                                        ops["blockscale_offsets"], q2, sf2)
+    torch.cuda.synchronize()
+    assert torch.equal(q, q2) and torch.equal(sf, sf2), f"fused epilogue, tile height {force_bm}"
+
+
 def test_mx_end_to_end_through_ops(esmoe):
     """quant -> GEMM through the Python entry points, compared like the reference's own test
     (calc_diff < 1e-3 against the unquantised product)."""
