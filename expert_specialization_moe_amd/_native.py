@@ -34,6 +34,8 @@ _sz = ctypes.c_size_t
 
 lib.esmoe_gemm_workspace_bytes.restype = _sz
 lib.esmoe_gemm_workspace_bytes.argtypes = [_i]
+lib.esmoe_stream_workspace.restype = _i
+lib.esmoe_stream_workspace.argtypes = [_vp, ctypes.POINTER(_vp), ctypes.POINTER(_sz)]
 lib.esmoe_fp8_blockwise_grouped_mm.restype = _i
 lib.esmoe_fp8_blockwise_grouped_mm.argtypes = [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]
 lib.esmoe_fp8_blockwise_grouped_mm_static.restype = _i

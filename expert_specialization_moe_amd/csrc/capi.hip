@@ -8,6 +8,8 @@
 #include <string.h>
 
 #include <mutex>
+#include <unordered_map>
+#include <vector>
 
 #include "esmoe.h"
 #include "gemm_args.h"
@@ -80,7 +82,7 @@ int current_device_info(DeviceInfo* out) {
 // ESMOE_* environment variables (tuning aids) are read once per process, on the first GEMM launch; a value the
 // kernels cannot honour is reported by every launch instead of being applied.
 struct Knobs {
-  int big_mt_fp8 = 12, big_mt_mx = 12, order = 0, light_share = -1, wgs_per_cu = 1, narrow_tail = -1;
+  int big_mt_fp8 = 12, big_mt_mx = 12, order = 0, light_share = -1, narrow_tail = -1, self_schedule = 1;
   char error[160] = "";
 };
 
@@ -103,8 +105,8 @@ const Knobs& knobs() {
     if (r.light_share < -1 || r.light_share > 32) snprintf(r.error, sizeof(r.error), "ESMOE_LIGHT_SHARE must be in [-1, 32]");
     r.narrow_tail = env_int("ESMOE_NARROW_TAIL", -1);
     if (r.narrow_tail < -1 || r.narrow_tail > 65536) snprintf(r.error, sizeof(r.error), "ESMOE_NARROW_TAIL must be in [-1, 65536]");
-    r.wgs_per_cu = env_int("ESMOE_WGS_PER_CU", 1);
-    if (r.wgs_per_cu < 1 || r.wgs_per_cu > 8) snprintf(r.error, sizeof(r.error), "ESMOE_WGS_PER_CU must be in [1, 8]");
+    r.self_schedule = env_int("ESMOE_SELF_SCHEDULE", 1);
+    if (r.self_schedule < 0 || r.self_schedule > 1) snprintf(r.error, sizeof(r.error), "ESMOE_SELF_SCHEDULE must be 0 or 1");
     return r;
   }();
   return k;
@@ -141,6 +143,47 @@ esmoe::SchedPolicy launch_policy(int force_bm, int kind) {
   return p;
 }
 
+// Schedule workspaces owned by the library, one per (device, stream) that has called a GEMM entry point without a
+// workspace.  They come out of chunks of kScratchSlots workspaces (room for ESMOE_MAX_EXPERTS experts each), zeroed
+// when the chunk is allocated; every launch leaves the counters of its workspace zero again (the last workgroup out
+// zeroes them), which is what lets those launches go without a schedule kernel.  A slot stays with its stream handle
+// for the life of the process.  Only a chunk allocation calls hipMalloc: the first call on a device, and the first
+// call of every kScratchSlots-th new stream after that.
+constexpr int kScratchSlots = 16;
+struct ScratchPool {
+  std::mutex mu;
+  std::unordered_map<hipStream_t, int32_t*> slot[64];   // by device
+  std::vector<int32_t*> free_slots[64];
+};
+ScratchPool g_pool;
+
+int library_scratch(hipStream_t stream, int32_t** ws, size_t* bytes) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail((int)err, "hipGetDevice failed: %s", hipGetErrorString(err));
+  if (dev < 0 || dev >= 64) return fail(ESMOE_ERR_UNSUPPORTED_DEVICE, "device index %d out of range", dev);
+  const size_t slot_bytes = esmoe_gemm_workspace_bytes(ESMOE_MAX_EXPERTS);
+  std::lock_guard<std::mutex> lock(g_pool.mu);
+  auto it = g_pool.slot[dev].find(stream);
+  if (it == g_pool.slot[dev].end()) {
+    if (g_pool.free_slots[dev].empty()) {
+      void* chunk = nullptr;
+      err = hipMalloc(&chunk, slot_bytes * kScratchSlots);
+      if (err == hipSuccess) err = hipMemset(chunk, 0, slot_bytes * kScratchSlots);
+      if (err != hipSuccess)
+        return fail((int)err, "allocating the library's schedule workspaces failed: %s (the first call on a device, and of a "
+                              "new stream once %d are in use, allocates: make it outside graph capture, or pass a workspace)",
+                    hipGetErrorString(err), kScratchSlots);
+      for (int i = kScratchSlots - 1; i >= 0; i--) g_pool.free_slots[dev].push_back((int32_t*)((char*)chunk + (size_t)i * slot_bytes));
+    }
+    it = g_pool.slot[dev].emplace(stream, g_pool.free_slots[dev].back()).first;
+    g_pool.free_slots[dev].pop_back();
+  }
+  *ws = it->second;
+  *bytes = slot_bytes;
+  return 0;
+}
+
 int check_common(const void* out, const void* a, const void* b, const int32_t* ps, const int32_t* eo, int num_experts,
                  int total_rows, int n, int k, int force_bm, void* workspace, size_t workspace_bytes, int out_dtype) {
   if (!out || !a || !b || !ps || !eo) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null tensor pointer");
@@ -154,24 +197,36 @@ int check_common(const void* out, const void* a, const void* b, const int32_t* p
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "out_dtype must be ESMOE_OUT_BF16 or ESMOE_OUT_FP16");
   if (force_bm != 0 && force_bm != 16 && force_bm != 32 && force_bm != 64 && force_bm != 128 && force_bm != 192)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "force_bm must be 0, 16, 32, 64, 128 or 192, got %d", force_bm);
-  if (!workspace || workspace_bytes < esmoe_gemm_workspace_bytes(num_experts))
-    return fail(ESMOE_ERR_WORKSPACE_TOO_SMALL, "workspace of %zu bytes is smaller than the %zu required",
-                workspace_bytes, esmoe_gemm_workspace_bytes(num_experts));
-  // (the kernel reads a schedule record with one 16-byte scalar load)
-  if ((uintptr_t)workspace % 16) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+  // (workspace == NULL with workspace_bytes == 0: the library's own workspace of the stream, resolved at the launch)
+  if (workspace || workspace_bytes) {
+    if (!workspace || workspace_bytes < esmoe_gemm_workspace_bytes(num_experts))
+      return fail(ESMOE_ERR_WORKSPACE_TOO_SMALL, "workspace of %zu bytes is smaller than the %zu required",
+                  workspace_bytes, esmoe_gemm_workspace_bytes(num_experts));
+    // (the kernel reads a schedule record with one 16-byte scalar load)
+    if ((uintptr_t)workspace % 16) return fail(ESMOE_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+  }
   if ((uintptr_t)a % 16 || (uintptr_t)b % 16 || (uintptr_t)out % 8)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "a and b must be 16-byte aligned, out 8-byte aligned");
   return 0;
 }
 
-int launch_gemm(esmoe::GemmArgs& g, int mx, int force_bm, void* stream) {
+// `owned`: g.ws is a workspace of the library (counters zero between launches), or null for the stream's own.
+int launch_gemm(esmoe::GemmArgs& g, int mx, int force_bm, void* stream, bool owned = false) {
   if (g.total_rows == 0) return 0;
   DeviceInfo info;
   int rc = current_device_info(&info);
   if (rc) return rc;
   if (knobs().error[0]) return fail(ESMOE_ERR_INVALID_ARGUMENT, "%s", knobs().error);
+  if (!g.ws) {
+    size_t bytes = 0;
+    rc = library_scratch((hipStream_t)stream, &g.ws, &bytes);
+    if (rc) return rc;
+    owned = true;
+  }
+  // One launch when the counters are known to be zero and a workgroup can rank the experts with a thread each.
+  g.self_schedule = owned && knobs().self_schedule && g.num_experts <= esmoe::kSelfScheduleMaxExperts;
   g.policy = launch_policy(force_bm, (mx ? 1 : 0) | (g.q_out ? 2 : 0));
-  int grid = info.cus * knobs().wgs_per_cu;
+  int grid = info.cus;   // one persistent workgroup per CU: its LDS ring takes the whole 160 KB
   rc = esmoe_launch_grouped_gemm(&g, mx, grid, (hipStream_t)stream);
   if (rc) return fail(rc, "grouped GEMM launch failed: %s", hipGetErrorString((hipError_t)rc));
   return 0;
@@ -180,6 +235,15 @@ int launch_gemm(esmoe::GemmArgs& g, int mx, int force_bm, void* stream) {
 }  // namespace
 
 extern "C" {
+
+int esmoe_stream_workspace(void* stream, void** workspace, size_t* bytes) {
+  g_err[0] = 0;
+  if (!workspace || !bytes) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null pointer");
+  int32_t* ws = nullptr;
+  int rc = library_scratch((hipStream_t)stream, &ws, bytes);
+  *workspace = ws;
+  return rc;
+}
 
 size_t esmoe_gemm_workspace_bytes(int num_experts) {
   if (num_experts < 0) num_experts = 0;
@@ -218,8 +282,17 @@ int esmoe_fp8_blockwise_grouped_mm_static(void* out, int out_dtype, const void* 
   if (num_experts > max_experts)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "the static workspace holds the schedule of at most %d experts, got %d",
                 max_experts, num_experts);
-  return esmoe_fp8_blockwise_grouped_mm(out, out_dtype, a, b, sa, sb, problem_sizes, expert_offsets, num_experts,
-                                        total_rows, n, k, force_bm, ws, ws_bytes, stream);
+  rc = check_common(out, a, b, problem_sizes, expert_offsets, num_experts, total_rows, n, k, force_bm, ws, ws_bytes, out_dtype);
+  if (rc) return rc;
+  if (!sa || !sb) return fail(ESMOE_ERR_INVALID_ARGUMENT, "null scale pointer");
+  esmoe::GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.b = b; g.sa = sa; g.sb = sb; g.out = out;
+  g.problem_sizes = problem_sizes; g.expert_offsets = expert_offsets;
+  g.ws = ws;
+  g.num_experts = num_experts; g.total_rows = total_rows; g.n = n; g.k = k; g.out_dtype = out_dtype;
+  // the static array is zero when the library is loaded and every launch leaves its counters zero
+  return launch_gemm(g, 0, force_bm, stream, /*owned=*/true);
 }
 
 int esmoe_fp8_blockwise_grouped_mm_swiglu_quant(void* q, float* scales, int mid_dtype, const void* a, const void* b,
@@ -554,6 +627,6 @@ int esmoe_host_decode_light(const int32_t* problem_sizes_host, const int32_t* ws
 
 const char* esmoe_last_error(void) { return g_err; }
 
-const char* esmoe_version(void) { return "esmoe 0.1 (gfx950)"; }
+const char* esmoe_version(void) { return "esmoe 0.3 (gfx950)"; }
 
 }  // extern "C"

@@ -26,6 +26,7 @@ struct GemmArgs {
   int n;
   int k;
   int out_dtype;        // 0 bf16, 1 fp16
+  int self_schedule;    // 1: no schedule kernel ran; ws counters are zero and every workgroup builds the records itself
   SchedPolicy policy;
 };
 

@@ -1124,6 +1124,7 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
       ws[kWsLightSplit] = split;
       ws[kWsLightTotal] = split + 2 * (items - split);
       ws[kWsLightCounter] = 0;
+      ws[kWsExitCounter] = 0;
       long heavy_cost = 0, light_cost = 0;
       for (int j = 0; j < num_experts; j++) {
         heavy_cost += s_cost[j][0];
@@ -1134,6 +1135,105 @@ __global__ void __launch_bounds__(1024) schedule_kernel(const int* __restrict__ 
     if (pos < kXcds) ws[ws_xcd_counter(pos)] = 0;
   }
   if (num_experts < kXcds && e >= num_experts && e < kXcds) ws[ws_xcd_counter(e)] = 0;
+}
+
+// The schedule built by the GEMM kernel itself (one launch per call; schedule.h, kSelfScheduleMaxExperts): every
+// workgroup does what schedule_kernel does, one thread per expert, with block-wide scans instead of that kernel's
+// per-thread loops (this runs in front of every workgroup's first tile), and writes the records into `ws`, where
+// the hand-out loop finds them with scalar loads.  All workgroups write the same values.  The launch constants are
+// returned instead of stored.  `lds` is the ring, free before the first tile.
+__device__ __forceinline__ void self_schedule(const GemmArgs& g, uint8_t* lds, int& hblocks, int& ltotal, int& lsplit, int& lshare) {
+  static_assert(kSelfScheduleMaxExperts <= kThreads, "one thread per expert");
+  int* s_m = (int*)lds;                         // rows by expert
+  int* s_blocks = s_m + kThreads;               // heavy blocks by schedule position
+  int* s_items = s_blocks + kThreads;           // light items by schedule position
+  int* s_wave = s_items + kThreads;             // per wavefront: blocks, items
+  long* s_cost = (long*)(s_wave + 2 * kWaves);  // per wavefront: heavy cost, light cost
+  const int E = g.num_experts, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const SchedPolicy policy = g.policy;
+  int* ws = g.ws;
+  int m = 0;
+  if (t < E) m = g.problem_sizes[t * 3];
+  if (m < 0) m = 0;
+  s_m[t] = m;
+  s_blocks[t] = 0;
+  s_items[t] = 0;
+  __syncthreads();
+  long hc = 0, lc = 0;
+  if (t < E) {
+    int pos = t;
+    if (policy.order != 1) {
+      pos = 0;
+      const int key = sched_order_key(m, policy);
+      for (int j = 0; j < E; j++) {
+        const int kj = sched_order_key(s_m[j], policy);
+        pos += (kj < key) || (kj == key && j < t);
+      }
+    }
+    ws[ws_rec(pos) + kRecExpert] = t;
+    ws[ws_rec(pos) + kRecRows] = m;
+    s_blocks[pos] = sched_heavy_blocks(m, g.n, policy);
+    s_items[pos] = sched_light_items(m, g.n, policy);
+    hc = sched_heavy_cost(m, g.n, policy);
+    lc = sched_light_cost(m, g.n, policy);
+  }
+  __syncthreads();
+  // exclusive prefix sums over the schedule positions (thread = position): inclusive scan inside the wavefront, then
+  // the totals of the wavefronts in front
+  const int b = s_blocks[t], it = s_items[t];
+  int sb = b, si = it;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int ub = __shfl_up(sb, d), ui = __shfl_up(si, d);
+    if (lane >= d) {
+      sb += ub;
+      si += ui;
+    }
+  }
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    hc += __shfl_xor(hc, d);
+    lc += __shfl_xor(lc, d);
+  }
+  if (lane == 63) {
+    s_wave[2 * wave] = sb;
+    s_wave[2 * wave + 1] = si;
+    s_cost[2 * wave] = hc;
+    s_cost[2 * wave + 1] = lc;
+  }
+  __syncthreads();
+  int blocks_before = 0, items_before = 0, blocks = 0, items = 0;
+  long heavy_cost = 0, light_cost = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; w++) {
+    const int wb = s_wave[2 * w], wi = s_wave[2 * w + 1];
+    if (w < wave) {
+      blocks_before += wb;
+      items_before += wi;
+    }
+    blocks += wb;
+    items += wi;
+    heavy_cost += s_cost[2 * w];
+    light_cost += s_cost[2 * w + 1];
+  }
+  if (t < E) {
+    ws[ws_rec(t) + kRecBlock] = blocks_before + sb - b;
+    ws[ws_rec(t) + kRecItem] = items_before + si - it;
+  }
+  if (t == 0) {
+    ws[ws_rec(E) + kRecBlock] = blocks;
+    ws[ws_rec(E) + kRecItem] = items;
+    ws[ws_rec(E) + kRecExpert] = -1;
+    ws[ws_rec(E) + kRecRows] = 0;
+  }
+  hblocks = __builtin_amdgcn_readfirstlane(blocks);
+  lsplit = __builtin_amdgcn_readfirstlane(sched_light_split(items, policy));
+  ltotal = __builtin_amdgcn_readfirstlane(lsplit + 2 * (items - lsplit));
+  lshare = __builtin_amdgcn_readfirstlane(sched_light_share(heavy_cost, light_cost, policy));
+  // the records are read back with scalar loads: every store of this workgroup has to be in L2 first.  (Also a
+  // compiler-visible full wait in front of the copy-pipelined K loops, which count their own copies.)
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
 }
 
 // Heights whose fp8-blockwise tiles run the hand-scheduled K block of gemm_tile_pp (bit 0: 128 rows, bit 1: 192 rows).
@@ -1155,8 +1255,15 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   __shared__ int s_item;
   __shared__ int s_counters[kXcds + 1];
   int* ws = g.ws;
-  const int hblocks = ws[kWsHeavyBlocks];
-  const int ltotal = ws[kWsLightTotal], lsplit = ws[kWsLightSplit];
+  int hblocks, ltotal, lsplit, lshare;
+  if (g.self_schedule) {
+    self_schedule(g, lds, hblocks, ltotal, lsplit, lshare);
+  } else {
+    hblocks = ws[kWsHeavyBlocks];
+    ltotal = ws[kWsLightTotal];
+    lsplit = ws[kWsLightSplit];
+    lshare = ws[kWsLightShare];
+  }
 #define ESMOE_CASE(MT_) \
   case (MT_): gemm_tile<MT_, MX, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
 
@@ -1165,7 +1272,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   // moves on to the other when its own is exhausted.
   const int xcd = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & (kXcds - 1);
   const int per_xcd = (int)gridDim.x / kXcds > 0 ? (int)gridDim.x / kXcds : 1;
-  const bool light_first = (int)(blockIdx.x / kXcds) * 32 / per_xcd >= 32 - ws[kWsLightShare];
+  const bool light_first = (int)(blockIdx.x / kXcds) * 32 / per_xcd >= 32 - lshare;
   int phase = 0, q = 0;
   // Queues known to be exhausted (bits 0-7: the XCDs' heavy queues, bit 8: the light items).  When a draw comes back
   // past the end of its queue and the launch has heavy blocks on every XCD, one look at all nine counters marks every
@@ -1309,6 +1416,17 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
 #endif
   }
 #undef ESMOE_CASE
+  // The last workgroup to leave zeroes the hand-out counters (nobody draws any more: every workgroup counts itself
+  // out after its last draw), so a workspace that held zero counters before the launch holds them again after it.
+  if (threadIdx.x == 0) {
+    const int left = atomicAdd(&ws[kWsExitCounter], 1);
+    if (left == (int)gridDim.x - 1) {
+#pragma unroll
+      for (int x = 0; x < kXcds; x++) __hip_atomic_store(&ws[ws_xcd_counter(x)], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&ws[kWsLightCounter], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&ws[kWsExitCounter], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
 }
 
 }  // namespace esmoe
@@ -1346,10 +1464,13 @@ extern "C" int esmoe_static_scratch(int32_t** ptr, size_t* bytes, int* max_exper
 
 extern "C" int esmoe_launch_grouped_gemm(const esmoe::GemmArgs* args, int mx, int grid, hipStream_t stream) {
   using namespace esmoe;
-  hipLaunchKernelGGL(schedule_kernel, dim3(1), dim3((args->num_experts + 63) & ~63), 0, stream, args->problem_sizes, args->num_experts, args->n,
-                     args->policy, args->ws);
-  hipError_t err = hipGetLastError();
-  if (err != hipSuccess) return (int)err;
+  if (args->self_schedule && args->num_experts > kSelfScheduleMaxExperts) return (int)hipErrorInvalidValue;
+  if (!args->self_schedule) {
+    hipLaunchKernelGGL(schedule_kernel, dim3(1), dim3((args->num_experts + 63) & ~63), 0, stream, args->problem_sizes, args->num_experts,
+                       args->n, args->policy, args->ws);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return (int)err;
+  }
   if (mx && args->q_out)
     hipLaunchKernelGGL((grouped_gemm_kernel<true, true>), dim3(grid), dim3(kThreads), 0, stream, *args);
   else if (mx)

@@ -192,6 +192,7 @@ constexpr int kWsLightTotal = 1;     // number of light tickets: whole items, th
 constexpr int kWsHeavyBlocks = 2;    // number of heavy blocks
 constexpr int kWsLightShare = 3;     // workgroups of every 32 that start on the light items
 constexpr int kWsLightSplit = 4;     // first light ticket that is a half item (sched_light_split)
+constexpr int kWsExitCounter = 16;   // workgroups of the launch that have left the hand-out loop: the last one zeroes every counter
 constexpr int kWsXcdCounter = 64;    // next heavy ticket of XCD x at word kWsXcdCounter + 32 * x (ws_xcd_counter)
 constexpr int kWsHeader = 64 + 32 * kXcds;   // then one record of kRecWords per schedule position, E + 1 of them
 // Record of schedule position p: first heavy block, first light item, expert index, rows (clamped at 0).
@@ -201,5 +202,11 @@ constexpr int kRecBlock = 0, kRecItem = 1, kRecExpert = 2, kRecRows = 3;
 ESMOE_HD int ws_xcd_counter(int xcd) { return kWsXcdCounter + 32 * xcd; }
 ESMOE_HD int ws_rec(int pos) { return kWsHeader + pos * kRecWords; }
 ESMOE_HD int ws_words(int num_experts) { return kWsHeader + (num_experts + 1) * kRecWords; }
+
+// One launch per call: when the counters of a workspace are known to be zero (a workspace the library owns: it is
+// zeroed when it is allocated, and the last workgroup to leave a launch zeroes the counters again), the GEMM kernel
+// needs no schedule kernel in front of it: every workgroup ranks the experts and builds the records itself, one
+// thread per expert, and writes them (the same values from every workgroup) for its own scalar loads.
+constexpr int kSelfScheduleMaxExperts = 512;
 
 }  // namespace esmoe

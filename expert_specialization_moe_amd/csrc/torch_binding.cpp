@@ -39,17 +39,10 @@ void check_rc(int rc, const char* op) { TORCH_CHECK(rc == 0, op, " failed (", rc
 
 int out_dtype_of(const torch::Tensor& t) { return t.scalar_type() == torch::kBFloat16 ? ESMOE_OUT_BF16 : ESMOE_OUT_FP16; }
 
-// Scratch for the device-built schedule: the caller's workspace when it is big
-// enough and aligned, otherwise a small tensor from the caching allocator.
-torch::Tensor schedule_scratch(const torch::Tensor* workspace, int64_t num_experts, const torch::Tensor& like) {
-  const int64_t need = (int64_t)esmoe_gemm_workspace_bytes((int)num_experts);
-  if (workspace && workspace->defined() && workspace->is_cuda() && workspace->device() == like.device() &&
-      workspace->is_contiguous() && workspace->nbytes() >= (size_t)need && (reinterpret_cast<uintptr_t>(workspace->data_ptr()) % 16) == 0) {
-    return *workspace;
-  }
-  return torch::empty({need}, torch::TensorOptions().dtype(torch::kUInt8).device(like.device()));
-}
-
+// Scratch for the device-built schedule: the operators pass no workspace to the library, which then uses its own
+// workspace of the current stream (zeroed once, left clean by every launch) and needs one launch per call instead of
+// two.  The `workspace` tensor of the reference's signature is accepted and not used: its contents are the caller's,
+// and a schedule built in it would need a kernel of its own in front of the GEMM to clear the counters.
 }  // namespace
 
 void es_fp8_blockwise_scaled_grouped_mm(torch::Tensor& output, const torch::Tensor& a, const torch::Tensor& b,
@@ -102,11 +95,10 @@ void es_fp8_blockwise_scaled_grouped_mm(torch::Tensor& output, const torch::Tens
   TORCH_CHECK(problem_sizes.is_contiguous() && expert_offsets.is_contiguous(), "metadata tensors must be contiguous");
   if (total_rows == 0) return;
   c10::DeviceGuard guard(a.device());
-  torch::Tensor ws = schedule_scratch(&workspace, num_experts, a);
   int rc = esmoe_fp8_blockwise_grouped_mm(
       output.data_ptr(), out_dtype_of(output), a.data_ptr(), b.data_ptr(), scales_a.data_ptr<float>(),
       scales_b.data_ptr<float>(), problem_sizes.data_ptr<int32_t>(), expert_offsets.data_ptr<int32_t>(),
-      (int)num_experts, (int)total_rows, (int)n, (int)k, /*force_bm=*/0, ws.data_ptr(), ws.nbytes(), current_stream(a));
+      (int)num_experts, (int)total_rows, (int)n, (int)k, /*force_bm=*/0, /*workspace=*/nullptr, 0, current_stream(a));
   check_rc(rc, "es_fp8_blockwise_scaled_grouped_mm");
 }
 
@@ -158,12 +150,10 @@ void es_fp8_blockwise_scaled_grouped_mm_swiglu_quant(torch::Tensor& quant_output
   TORCH_CHECK(problem_sizes.is_contiguous() && expert_offsets.is_contiguous(), "metadata tensors must be contiguous");
   if (total_rows == 0) return;
   c10::DeviceGuard guard(a.device());
-  torch::Tensor ws = schedule_scratch(&workspace, num_experts, a);
   int rc = esmoe_fp8_blockwise_grouped_mm_swiglu_quant(
       quant_output.data_ptr(), scales_out.data_ptr<float>(), mid_dtype_bf16 ? ESMOE_OUT_BF16 : ESMOE_OUT_FP16, a.data_ptr(),
       b.data_ptr(), scales_a.data_ptr<float>(), scales_b.data_ptr<float>(), problem_sizes.data_ptr<int32_t>(),
-      expert_offsets.data_ptr<int32_t>(), (int)num_experts, (int)total_rows, (int)n, (int)k, /*force_bm=*/0, ws.data_ptr(),
-      ws.nbytes(), current_stream(a));
+      expert_offsets.data_ptr<int32_t>(), (int)num_experts, (int)total_rows, (int)n, (int)k, /*force_bm=*/0, /*workspace=*/nullptr, 0, current_stream(a));
   check_rc(rc, "es_fp8_blockwise_scaled_grouped_mm_swiglu_quant");
 }
 
@@ -217,12 +207,11 @@ void es_sm100_mxfp8_blockscaled_grouped_mm(const torch::Tensor& a, const torch::
               "metadata tensors must be contiguous");
   if (total_rows == 0) return;
   c10::DeviceGuard guard(a.device());
-  torch::Tensor ws = schedule_scratch(nullptr, num_experts, a);
   int rc = esmoe_mxfp8_grouped_mm(d.data_ptr(), out_dtype_of(d), a.data_ptr(), b.data_ptr(),
                                   (const uint8_t*)sfa.data_ptr(), (const uint8_t*)sfb.data_ptr(),
                                   problem_sizes.data_ptr<int32_t>(), expert_offsets.data_ptr<int32_t>(),
                                   blockscale_offsets.data_ptr<int32_t>(), (int)num_experts, (int)total_rows, (int)n,
-                                  (int)k, /*force_bm=*/0, ws.data_ptr(), ws.nbytes(), current_stream(a));
+                                  (int)k, /*force_bm=*/0, /*workspace=*/nullptr, 0, current_stream(a));
   check_rc(rc, "es_sm100_mxfp8_blockscaled_grouped_mm");
 }
 
@@ -275,12 +264,11 @@ void es_mxfp8_blockscaled_grouped_mm_swiglu_quant(torch::Tensor& quant_output, t
               "metadata tensors must be contiguous");
   if (total_rows == 0) return;
   c10::DeviceGuard guard(a.device());
-  torch::Tensor ws = schedule_scratch(nullptr, num_experts, a);
   int rc = esmoe_mxfp8_grouped_mm_swiglu_quant(
       quant_output.data_ptr(), (uint8_t*)scale_factor.data_ptr(), mid_dtype_bf16 ? ESMOE_OUT_BF16 : ESMOE_OUT_FP16,
       a.data_ptr(), b.data_ptr(), (const uint8_t*)sfa.data_ptr(), (const uint8_t*)sfb.data_ptr(),
       problem_sizes.data_ptr<int32_t>(), expert_offsets.data_ptr<int32_t>(), blockscale_offsets.data_ptr<int32_t>(),
-      (int)num_experts, (int)total_rows, (int)sf_rows, (int)n, (int)k, /*force_bm=*/0, ws.data_ptr(), ws.nbytes(),
+      (int)num_experts, (int)total_rows, (int)sf_rows, (int)n, (int)k, /*force_bm=*/0, /*workspace=*/nullptr, 0,
       current_stream(a));
   check_rc(rc, "es_mxfp8_blockscaled_grouped_mm_swiglu_quant");
 }

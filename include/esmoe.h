@@ -35,10 +35,31 @@ extern "C" {
 
 #define ESMOE_MAX_EXPERTS 1024 /* same limit as the reference, es_fp8_blockwise_launcher.cuh:53 */
 
-/* Bytes of device scratch the two GEMM entry points need for `num_experts` experts
- * (the device-built tile schedule and its work counter).  The scratch must be 16-byte aligned (device allocations are);
- * its contents before a call do not matter. */
+/* ABI revision of this header; esmoe_version() of a matching library reads "esmoe 0.<ESMOE_ABI> (gfx950)".
+ * 3: a null `workspace` selects the library's own; esmoe_stream_workspace added; the workspace layout gained an exit
+ *    counter (same size).  2: the esmoe_host_* mirrors gained `kind` after `force_bm`; esmoe_gemm_workspace_bytes
+ *    grew from 16 E + 80 to 16 E + 1296 bytes and the workspace must be 16-byte aligned. */
+#define ESMOE_ABI 3
+
+/* Bytes of device scratch the GEMM entry points need for `num_experts` experts
+ * (the device-built tile schedule and its hand-out counters).  The scratch must be 16-byte aligned (device allocations
+ * are); its contents before a call do not matter: a one-workgroup schedule kernel in front of the GEMM kernel writes
+ * every word the GEMM kernel reads.
+ *
+ * Every GEMM entry point below also accepts workspace == NULL with workspace_bytes == 0: the library then uses a
+ * workspace of its own, one per (device, stream), whose counters it knows to be zero between launches (zeroed when
+ * allocated; the last workgroup of every launch zeroes them again).  Such a call is ONE kernel launch: every workgroup
+ * builds the schedule records itself (up to 512 experts; more fall back to the schedule kernel).  This replaces the
+ * reference's pre-compute launch and its twelve per-call scratch tensors (es_fp8_blockwise_launcher.cuh:18-86,
+ * es_fp8_blockwise.cu:58-75) by nothing.  The library's workspaces are allocated 16 at a time (hipMalloc + hipMemset):
+ * by the first such call on a device, and again by the first call of a 17th, 33rd, ... distinct stream handle; those
+ * calls must not happen during graph capture.  A slot stays with its stream handle until the process ends; calls on
+ * one stream are ordered and safe, a graph captured on a stream keeps that stream's workspace. */
 size_t esmoe_gemm_workspace_bytes(int num_experts);
+
+/* The library's own schedule workspace of `stream` on the current device (allocated on first use, see above), for
+ * tools and tests that inspect the schedule records a launch left there.  No counterpart in the reference. */
+int esmoe_stream_workspace(void* stream, void** workspace, size_t* bytes);
 
 /*
  * FP8-blockwise scaled grouped GEMM.
@@ -69,7 +90,9 @@ int esmoe_fp8_blockwise_grouped_mm(void* out, int out_dtype, const void* a, cons
  * results.  No counterpart in the reference, whose operator allocates its scratch tensors on every call
  * (es_fp8_blockwise.cu:58-75).  The schedule workspace is a static array inside the library, one copy per GPU,
  * ESMOE_STATIC_MAX_EXPERTS experts at most (more are rejected with ESMOE_ERR_INVALID_ARGUMENT); the call allocates
- * and frees nothing.  All calls on one GPU share that array: calls that overlap in time on one GPU (two streams,
+ * and frees nothing.  The array is zero when the library is loaded and every launch leaves its counters zero, so up to
+ * 512 experts the call is one kernel launch.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress) and reads the device's properties: make it outside graph capture.  All calls on one GPU share that array: calls that overlap in time on one GPU (two streams,
  * two threads) race on it and must be serialised by the caller; calls ordered on one stream are safe.
  */
 #define ESMOE_STATIC_MAX_EXPERTS 1024

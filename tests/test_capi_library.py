@@ -47,4 +47,9 @@ def test_argument_validation_needs_no_gpu(esmoe):
     assert rc == -1 and "in_dtype" in _native.last_error()
     rc = lib.esmoe_mxfp8_grouped_quant(p, 0, p, p, p, p, p, 4, 10, 100, 128, None)
     assert rc == -1 and "sf_rows" in _native.last_error()
-    assert lib.esmoe_version().startswith(b"esmoe")
+    # a size without a pointer is not the "library's own workspace" form (null pointer AND zero bytes)
+    rc = lib.esmoe_fp8_blockwise_grouped_mm(p, 0, p, p, p, p, p, p, 4, 10, 128, 128, 0, None, 4096, None)
+    assert rc == -2 and "workspace" in _native.last_error()
+    header = open(os.path.join(ROOT, "include", "esmoe.h")).read()
+    abi = int(re.search(r"#define ESMOE_ABI (\d+)", header).group(1))
+    assert lib.esmoe_version() == f"esmoe 0.{abi} (gfx950)".encode()
