@@ -373,6 +373,7 @@ int grouped_quant_common(const void* in, int in_dtype, const int32_t* problem_si
   if (num_experts < 1 || num_experts > ESMOE_MAX_EXPERTS)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "num_experts must be in [1, %d], got %d", ESMOE_MAX_EXPERTS, num_experts);
   if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must align to 128, got %d", k);
+  if (k > (1 << 20)) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must be <= 1048576, got %d", k);
   if (in_dtype != ESMOE_IN_BF16 && in_dtype != ESMOE_IN_FP16)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "in_dtype must be ESMOE_IN_BF16 or ESMOE_IN_FP16");
   if (total_rows < 0 || sf_rows < 0 || sf_rows % 128)
@@ -380,7 +381,7 @@ int grouped_quant_common(const void* in, int in_dtype, const int32_t* problem_si
   if ((uintptr_t)in % 16 || (uintptr_t)q % 8 || (uintptr_t)sf % 16)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "in and sf must be 16-byte aligned, q 8-byte aligned");
   if (total_rows == 0 || sf_rows == 0) return 0;
-  if (sf_rows / 128 > 65535)   // one workgroup row per 128 scale rows, in the y dimension of the launch
+  if (sf_rows / 128 > 65535)   // keeps the launch's workgroup count (32 rows x 256 columns each) far inside 2^31
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "sf_rows must not exceed 65535 * 128, got %d", sf_rows);
   DeviceInfo info;
   int rc = current_device_info(&info);
@@ -410,6 +411,7 @@ int esmoe_swiglu_mxfp8_grouped_quant(const void* in, int in_dtype, const int32_t
 int esmoe_mxfp8_quant_weight(const void* in, int in_dtype, void* q, uint8_t* sf, long rows, int k, void* stream) {
   g_err[0] = 0;
   if (k <= 0 || k % 128) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must align to 128, got %d", k);
+  if (k > (1 << 20)) return fail(ESMOE_ERR_INVALID_ARGUMENT, "k must be <= 1048576, got %d", k);
   if (in_dtype != ESMOE_IN_BF16 && in_dtype != ESMOE_IN_FP16)
     return fail(ESMOE_ERR_INVALID_ARGUMENT, "in_dtype must be ESMOE_IN_BF16 or ESMOE_IN_FP16");
   if (rows < 0 || rows % 128 || rows / 128 > 65535)

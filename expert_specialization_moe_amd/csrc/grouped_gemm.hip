@@ -782,8 +782,13 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int erow,
     const int grow = trow > a_last ? a_last : trow;
     vs[q] = (uint32_t)grow * (uint32_t)KB * 4 + ((lane & 3) < KB ? (lane & 3) : KB - 1) * 4;
   }
+#ifdef ESMOE_EXP_SAMEPANEL   // timing experiment (results wrong): every tall tile of an expert reads the same operand panels
+  const uint8_t* a_ptr = (const uint8_t*)g.a + (row_base + 0) * K - kBias;
+  const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + 0) * K - kBias;
+#else
   const uint8_t* a_ptr = (const uint8_t*)g.a + (row_base + m0) * K - kBias;
   const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + (FUSE ? 0 : n0)) * K - kBias;
+#endif
   const uint8_t* sa_ptr = (const uint8_t*)(g.sa + (row_base + m0) * KB);
   const uint32_t t_dst = lds0 + kTBase + grp * 2 * kTSlot + wj * kTCopies * 1024;   // + slot * kTSlot
   const uint32_t w_dst = lds0 + wave * 4096;                                        // + slot * kWSlot

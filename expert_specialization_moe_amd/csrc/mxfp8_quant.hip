@@ -7,13 +7,22 @@
 // amax (448 = 1.75 * 2^8  =>  E = exponent(amax) - 8 + (mantissa > .75)), which equals
 // the reference's float route with a correctly rounded 1/448.
 //
-// Work decomposition: one workgroup per 128 rows of the *scale* row space
-// (blockscale_offsets are multiples of 128, so the rows belong to one expert) x 256
-// columns (128 in the SwiGLU form).  32 (16) lanes read one row segment (16 bytes each,
-// a 512-byte coalesced segment), 4 lanes share one 32-wide block and reduce amax with
-// two lane swaps.  The 512-byte scale tiles (128 rows x 4 scale columns, layout
-// ((32,4),4):((16,4),1), group_quant.cuh:25; tiles of consecutive 128-column blocks are
-// consecutive in memory) are assembled in LDS and written with 16-byte stores.
+// Work decomposition.  A 512-byte scale tile (128 rows x 4 scale columns, layout ((32,4),4):((16,4),1),
+// group_quant.cuh:25) keeps the four scale bytes of row r (one dword per 128 columns) at (r % 32) * 16 + (r / 32) * 4:
+// rows r, r + 32, r + 64 and r + 96 of a tile share one 16-byte unit, and eight neighbouring rows a 128-byte line.
+// Scale bytes that reach memory as scattered dwords cost 4 us of 31 on 8192 x 7168 rows (lines that are filled piece by
+// piece from several L2s; one store instruction instead of four for the same dwords changes nothing); whole units
+// side by side cost a tenth of that.  (Flat 4 KB runs of consecutive rows per load instruction, the shape of the FP8
+// 1x128 quantiser of fp8_quant.hip, would stream 8 % faster than 512-byte row segments, but their scale bytes can only
+// leave as scattered dwords; 16-byte units from rows 32 apart with 4 KB runs lose the gain to the row stride.)
+// So a workgroup of 256 threads takes the rows
+// {s * 8 + i + 32 * j : i < 8, j < 4} of one 128-row slab of the *scale* row space (blockscale_offsets are multiples of
+// 128: a slab belongs to one expert) x 256 columns (128 in the SwiGLU form): 32 (16) lanes read one 512-byte row
+// segment, 8 (16) rows per pass, one pass per quarter j, four (SwiGLU: two, of two loads) 16-byte loads in flight
+// per lane; 4 lanes share one 32-wide block and reduce amax with two lane swaps, the four codes of a row's 128-column
+// group are gathered with two more, and after the passes the group's first lane holds the row's whole 16-byte unit:
+// the workgroup writes whole 128-byte lines of the scale tiles.  Rows between the expert's last row and the end of
+// its last 128-row tile get scale bytes 0 (the reference leaves them unspecified).
 //
 // Two more forms of the same kernel (no counterpart in the reference, which quantises weights by passing
 // the activation operator a transposed problem list, test/test_es_sm100_mxfp8_blockscaled_grouped_quant.py:53,87-96,
@@ -33,11 +42,9 @@ namespace esmoe {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 
-// A workgroup covers 128 rows x 256 columns (32 lanes per row segment, 16 rows per pass, 512 threads): 512-byte row
-// segments stream 8 % faster than 256-byte ones on the large inputs.  The SwiGLU form, whose inputs are small and whose
-// lanes hold twice the registers, keeps 128 columns and 256 threads.
-template <bool SWIGLU> constexpr int quant_cols() { return SWIGLU ? 128 : 256; }
-template <bool SWIGLU> constexpr int quant_threads() { return quant_cols<SWIGLU>() * 2; }
+// (measured on 8192 x 7168 rows: 128 ... 1024 columns per workgroup of 256 or 512 threads are within 1 % of one another)
+template <bool SWIGLU> constexpr int quant_cols() { return SWIGLU ? 128 : 256; }   // columns per workgroup
+template <bool SWIGLU> constexpr int quant_threads() { return 256; }
 
 template <bool FP16>
 __device__ __forceinline__ void unpack8(v4i raw, float* x) {
@@ -60,17 +67,23 @@ __device__ __forceinline__ float round_to_input_type(float h) {
   else return (float)(__bf16)h;
 }
 
+// Value of another lane through DPP (inside the VALU, no LDS trip).  CTRL 0xB1 / 0x4E: lane ^ 1 / lane ^ 2 inside
+// each group of four; 0x100 + n: lane + n inside each row of 16 lanes (0 from past the row's end).
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) { return __builtin_bit_cast(float, dpp_i32<CTRL>(__builtin_bit_cast(int, v))); }
+
 template <bool FP16, bool SWIGLU>
-__global__ void __launch_bounds__(quant_threads<SWIGLU>()) __attribute__((amdgpu_waves_per_eu(SWIGLU ? 4 : 6, 8))) mxfp8_quant_kernel(const uint16_t* __restrict__ in,
-                                                                    const int* __restrict__ problem_sizes,
-                                                                    const int* __restrict__ expert_offsets,
-                                                                    const int* __restrict__ blockscale_offsets,
-                                                                    uint8_t* __restrict__ q, uint8_t* __restrict__ sf,
-                                                                    int num_experts, int k, long dense_rows) {
-  constexpr int kCols = quant_cols<SWIGLU>(), kLanes = kCols / 8, kTiles = kCols / 128;
-  __shared__ __attribute__((aligned(16))) uint8_t s_sf[512 * kTiles];   // the 512-byte scale tiles of the workgroup's columns
-  const int kt = blockIdx.x;               // tile of kCols columns (the last one may be 128 wide)
-  const int sf_row0 = blockIdx.y * 128;    // first row of this tile in scale-row space
+__global__ void __launch_bounds__(quant_threads<SWIGLU>()) __attribute__((amdgpu_waves_per_eu(6, 8))) mxfp8_quant_kernel(
+    const uint16_t* __restrict__ in, const int* __restrict__ problem_sizes, const int* __restrict__ expert_offsets,
+    const int* __restrict__ blockscale_offsets, uint8_t* __restrict__ q, uint8_t* __restrict__ sf, int num_experts, int k,
+    long dense_rows, int ktiles) {
+  constexpr int kCols = quant_cols<SWIGLU>(), kLanes = kCols / 8, kRowsPerPass = quant_threads<SWIGLU>() / kLanes, kSubs = 32 / kRowsPerPass;
+  // consecutive workgroups: consecutive column tiles of the same rows, then the next rows of the slab
+  const int kt = blockIdx.x % ktiles;                                       // tile of kCols columns (the last one may be 128 wide)
+  const int s = (blockIdx.x / ktiles) % kSubs;
+  const int sf_row0 = (int)((long)(blockIdx.x / (ktiles * kSubs)) * 128);   // first row of the slab in scale-row space
   const int tid = threadIdx.x;
 
   int m_e, r0;
@@ -81,73 +94,81 @@ __global__ void __launch_bounds__(quant_threads<SWIGLU>()) __attribute__((amdgpu
     row_base = 0;
     sf_base = 0;
   } else {
-    // expert owning scale row sf_row0: last e with blockscale_offsets[e] <= sf_row0
-    int lo = 0, hi = num_experts;
-    while (hi - lo > 1) {
-      int mid = (lo + hi) >> 1;
-      if (blockscale_offsets[mid] <= sf_row0) lo = mid; else hi = mid;
+    // expert owning scale row sf_row0: the last e with blockscale_offsets[e] <= sf_row0 (the offsets never decrease),
+    // counted by the wavefront 64 offsets at a time: one trip to memory where a bisection makes one per step
+    int cnt = 0;
+    for (int base = 0; base < num_experts; base += 64) {
+      const int idx = base + (tid & 63);
+      const int b = idx < num_experts ? blockscale_offsets[idx] : 0x7fffffff;
+      cnt += __popcll(__ballot(b <= sf_row0));
     }
-    const int e = lo;
+    const int e = __builtin_amdgcn_readfirstlane(cnt) - 1;
+    if (e < 0) return;
     m_e = problem_sizes[e * 3];
-    r0 = sf_row0 - blockscale_offsets[e];  // first row of the tile inside the expert
+    if (m_e < 0) m_e = 0;
+    r0 = sf_row0 - blockscale_offsets[e];  // first row of the slab inside the expert
     row_base = expert_offsets[e];
     sf_base = blockscale_offsets[e];
   }
-  if (r0 < 0 || r0 >= m_e) return;           // tile past the expert's rows: nothing defined there
-  const int kcols = k >> 5;
-  const long in_stride = SWIGLU ? 2L * k : k;   // SwiGLU reads [rows, 2K]: gate | up
-
+  // slabs past the expert's rows (an empty expert has none; the launch's scale rows may run past the last expert's)
+  if (r0 < 0 || r0 >= m_e) return;
   const int sub = tid % kLanes;    // 16-byte column of the row segment: elements [8*sub, 8*sub + 8)
-  const int rrow = tid / kLanes;   // row within a 16-row pass
+  const int rrow = tid / kLanes;   // row within a pass
   const bool col_ok = kt * kCols + sub * 8 < k;
-  v4i raw[8], rup[SWIGLU ? 8 : 1];
+  // wave-uniform 64-bit bases, 32-bit lane offsets (SwiGLU reads [rows, 2K]: gate | up)
+  const uint32_t row_pitch = (SWIGLU ? 2u : 1u) * (uint32_t)k * 2u;   // bytes
+  const char* const in_b = (const char*)(in + (row_base + r0) * (SWIGLU ? 2L * k : (long)k) + kt * kCols);
+  uint8_t* const q_b = q + (row_base + r0) * (long)k + kt * kCols;
+  const int rl0 = s * kRowsPerPass + rrow;   // this lane's row of quarter 0; quarter j: + 32 j
+
+  v4i raw[4], rup[SWIGLU ? 4 : 1];
 #pragma unroll
-  for (int p = 0; p < 8; p++) {
-    int r = r0 + p * 16 + rrow;
-    raw[p] = v4i{0, 0, 0, 0};
-    if constexpr (SWIGLU) rup[p] = v4i{0, 0, 0, 0};
-    if (r < m_e && col_ok) {
-      const uint16_t* src = in + (row_base + r) * in_stride + kt * kCols + sub * 8;
-      raw[p] = __builtin_nontemporal_load((const v4i*)src);
-      if constexpr (SWIGLU) rup[p] = __builtin_nontemporal_load((const v4i*)(src + k));
+  for (int j = 0; j < 4; j++) {
+    const int rl = rl0 + 32 * j;
+    raw[j] = v4i{0, 0, 0, 0};
+    if constexpr (SWIGLU) rup[j] = v4i{0, 0, 0, 0};
+    if (r0 + rl < m_e && col_ok) {
+      const char* src = in_b + (uint32_t)rl * row_pitch + sub * 16;
+      raw[j] = __builtin_nontemporal_load((const v4i*)src);
+      if constexpr (SWIGLU) rup[j] = __builtin_nontemporal_load((const v4i*)(src + 2 * (uint32_t)k));
     }
   }
+  v4i unit;   // the 16-byte unit of row rl0, 128-column group sub / 16 (in the group's first lane)
 #pragma unroll
-  for (int p = 0; p < 8; p++) {
-    const int rt = p * 16 + rrow;  // row within the tile
-    const int r = r0 + rt;
+  for (int j = 0; j < 4; j++) {
+    const int rl = rl0 + 32 * j;
+    const bool live = r0 + rl < m_e && col_ok;
     float x[8];
-    unpack8<FP16>(raw[p], x);
+    unpack8<FP16>(raw[j], x);
     if constexpr (SWIGLU) {
-      float u[8];
-      unpack8<FP16>(rup[p], u);
+      float up[8];
+      unpack8<FP16>(rup[j], up);
 #pragma unroll
-      for (int i = 0; i < 8; i++) x[i] = round_to_input_type<FP16>(swiglu_f32(x[i], u[i]));
+      for (int t = 0; t < 8; t++) x[t] = round_to_input_type<FP16>(swiglu_f32(x[t], up[t]));
     }
     float amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; i++) amax = __builtin_fmaxf(amax, __builtin_fabsf(x[i]));
-    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 1));
-    amax = __builtin_fmaxf(amax, __shfl_xor(amax, 2));
+    for (int t = 0; t < 8; t++) amax = __builtin_fmaxf(amax, __builtin_fabsf(x[t]));
+    amax = __builtin_fmaxf(amax, dpp_f32<0xB1>(amax));   // lane ^ 1
+    amax = __builtin_fmaxf(amax, dpp_f32<0x4E>(amax));   // lane ^ 2
     const int code = mx_scale_code(amax);
     const float inv = mx_scale_inverse(amax, code);
-    float y[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) y[i] = __builtin_amdgcn_fmed3f(x[i] * inv, -448.f, 448.f);
-    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], 0, false);
-    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
-    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], 0, false);
-    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
-    if (r < m_e && col_ok) {
-      __builtin_nontemporal_store(v2i{w0, w1}, (v2i*)(q + (row_base + r) * k + kt * kCols + sub * 8));
-    }
-    if ((sub & 3) == 0) s_sf[(sub >> 4) * 512 + (rt & 31) * 16 + (rt >> 5) * 4 + ((sub >> 2) & 3)] = (uint8_t)(r < m_e ? code : 0);
+    // |x| * inv <= 448 for every finite input (the scale is the smallest power of two >= amax / 448), so the
+    // conversion needs no clamp
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(x[0] * inv, x[1] * inv, 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(x[2] * inv, x[3] * inv, w0, true);
+    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(x[4] * inv, x[5] * inv, 0, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(x[6] * inv, x[7] * inv, w1, true);
+    if (live) __builtin_nontemporal_store(v2i{w0, w1}, (v2i*)(q_b + (long)rl * k + sub * 8));
+    // 16 consecutive lanes hold the row's four blocks of a 128-column scale tile: their codes -> one dword in the
+    // first of them (rows past the expert's last: 0, loaded as zeros)
+    int codes = live ? code : 0;
+    codes |= dpp_i32<0x104>(codes) << 8;     // from lane + 4 of the 16-lane row
+    codes |= dpp_i32<0x108>(codes) << 16;    // from lane + 8
+    unit[j] = codes;
   }
-  __syncthreads();
-  if (tid < 32 * kTiles && kt * kTiles + (tid >> 5) < (k >> 7)) {   // consecutive 128-column tiles are consecutive 512-byte tiles
-    uint8_t* dst = sf + sf_base * kcols + ((long)(r0 >> 7) * (k >> 7) + kt * kTiles) * 512;
-    *(v4i*)(dst + tid * 16) = *(const v4i*)(s_sf + tid * 16);
-  }
+  if ((sub & 15) == 0 && col_ok)
+    *(v4i*)(sf + sf_base * (k >> 5) + ((long)(r0 >> 7) * (k >> 7) + kt * (kCols / 128) + (sub >> 4)) * 512 + rl0 * 16) = unit;
 }
 
 }  // namespace esmoe
@@ -158,12 +179,16 @@ extern "C" int esmoe_launch_mxfp8_quant(const void* in, int in_dtype, const int*
                                         int num_experts, long sf_rows, int k, int swiglu, long dense_rows,
                                         hipStream_t stream) {
   using namespace esmoe;
-  const unsigned rows128 = (unsigned)(sf_rows / 128);
-  if (k < 128 || rows128 == 0) return 0;
+  const long slabs = sf_rows / 128;
+  if (k < 128 || slabs == 0) return 0;
 #define ESMOE_LAUNCH_QUANT(F16_, SW_)                                                                               \
-  hipLaunchKernelGGL((mxfp8_quant_kernel<F16_, SW_>), dim3((k + quant_cols<SW_>() - 1) / quant_cols<SW_>(), rows128), \
-                     dim3(quant_threads<SW_>()), 0, stream, (const uint16_t*)in,                                   \
-                     problem_sizes, expert_offsets, blockscale_offsets, (uint8_t*)q, sf, num_experts, k, dense_rows)
+  do {                                                                                                              \
+    const int ktiles = (k + quant_cols<SW_>() - 1) / quant_cols<SW_>();                                             \
+    const int subs = 32 / (quant_threads<SW_>() / (quant_cols<SW_>() / 8));                                         \
+    hipLaunchKernelGGL((mxfp8_quant_kernel<F16_, SW_>), dim3((unsigned)(slabs * subs * ktiles)), dim3(quant_threads<SW_>()), 0, \
+                       stream, (const uint16_t*)in, problem_sizes, expert_offsets, blockscale_offsets, (uint8_t*)q, sf, \
+                       num_experts, k, dense_rows, ktiles);                                                          \
+  } while (0)
   if (in_dtype == 1) {
     if (swiglu) ESMOE_LAUNCH_QUANT(true, true); else ESMOE_LAUNCH_QUANT(true, false);
   } else {
