@@ -226,6 +226,10 @@ int launch_gemm(esmoe::GemmArgs& g, int mx, int force_bm, void* stream, bool own
   // One launch when the counters are known to be zero and a workgroup can rank the experts with a thread each.
   g.self_schedule = owned && knobs().self_schedule && g.num_experts <= esmoe::kSelfScheduleMaxExperts;
   g.policy = launch_policy(force_bm, (mx ? 1 : 0) | (g.q_out ? 2 : 0));
+  // every height the schedule can hand out must be one the kernel has a tile function for (it has no other case)
+  if ((g.policy.force_mt && !esmoe::sched_valid_mt(g.policy.force_mt)) || (g.policy.big_mt != 8 && g.policy.big_mt != 12))
+    return fail(ESMOE_ERR_INVALID_ARGUMENT, "tile heights %d / %d rows are not compiled into the kernels",
+                g.policy.force_mt * 16, g.policy.big_mt * 16);
   int grid = info.cus;   // one persistent workgroup per CU: its LDS ring takes the whole 160 KB
   rc = esmoe_launch_grouped_gemm(&g, mx, grid, (hipStream_t)stream);
   if (rc) return fail(rc, "grouped GEMM launch failed: %s", hipGetErrorString((hipError_t)rc));

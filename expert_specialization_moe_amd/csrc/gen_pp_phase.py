@@ -38,26 +38,11 @@ promotions follow the barrier; a fragment buffer is overwritten by a read that i
 the last one that used it, and LDS data returns much later than an MFMA reads its operands; s_nop 0 separates
 a write of m0 from the copy that uses it.
 """
-import sys
 
 NT = 4
-ABLATE = set()   # timing experiments only (results wrong): "fma", "copy" ("copyw", "copyt", "copys": weight, token, scale copies only), "roll", "read", "scread", "barrier", "vmwait";
-                 # "bookodd": bookkeeping behind every second MFMA instead (results right);
-                 # "prioN" / "mprioN": the matrix / memory phase at wave priority N ("prio0": none; results right);
-                 # "latebar": every LDS read of the memory phase waited for in front of its barrier (results right)
-
-
 MATRIX_PRIO = 3   # wave priority during the matrix phase (the memory phase runs at 0): where both wavefronts of a SIMD
                   # have an instruction ready, the one that feeds the matrix core goes first (one large expert,
                   # 12288 x 4096 x 7168: MXFP8 -1.7 %, FP8-blockwise -0.6 %; the memory phase first instead: +1.7 %, +0.3 %)
-
-
-def prio(word, default=None):
-    """Wave priority asked for by an ablation word such as "prio2" / "mprio3" (matrix / memory phase), else `default`."""
-    for a in ABLATE:
-        if a.startswith(word) and a[len(word):].isdigit():
-            return int(a[len(word):])
-    return default
 
 
 def with_prio(lines, level, before):
@@ -145,7 +130,7 @@ def memory_phase(p):
     # its own wavefronts refill after the barrier that ends the matrix phase, and every wavefront of the group has
     # waited for these reads before it gets there.  So the barrier is not kept waiting for them
     # (one large expert, 12288 x 4096 x 7168 FP8-blockwise: -3.4 %).
-    L.append("s_waitcnt lgkmcnt(0)" if "latebar" in ABLATE else f"s_waitcnt lgkmcnt({4 + len(sr)})")
+    L.append(f"s_waitcnt lgkmcnt({4 + len(sr)})")
     L.append(f"s_waitcnt vmcnt({p.ntc + 5}) ; explicit")
     L.append("s_barrier")
     L.append("s_waitcnt lgkmcnt(0)")
@@ -180,7 +165,7 @@ def matrix_phase(p):
     L = []
     total = p.mtw * NT
     lag = 3
-    atoms, late = bookkeeping(p) if "nobook" not in ABLATE else ([], [])
+    atoms, late = bookkeeping(p)
     last_roll = (p.mtw - 3) * NT      # MFMA behind which the last rolling token read issues
     for j in range(total):
         mt, nt = divmod(j, NT)
@@ -195,10 +180,7 @@ def matrix_phase(p):
             L += promotion(p, j - lag)
         # bookkeeping behind the first three MFMAs, which have no promotions to issue yet (two groups each); the
         # token-slot group once the last rolling read has used al and ah
-        if "bookodd" in ABLATE:
-            if j >= 1 and atoms and j % 2 == 1:
-                L += atoms.pop(0)
-        elif j < lag:
+        if j < lag:
             for _ in range(2):
                 if atoms:
                     L += atoms.pop(0)
@@ -223,40 +205,9 @@ def print_body(name, lines):
             print('  "%s%s"%s' % (l, "" if last else "\\n\\t", "" if last else " \\"))
 
 
-def ablated(lines):
-    out = []
-    for l in lines:
-        if "fma" in ABLATE and l.startswith("v_fmac"):
-            continue
-        if "halffma" in ABLATE and l.startswith("v_fmac") and l.split("]")[0][-1] in "13":
-            continue
-        if "copy" in ABLATE and l.startswith("global_load_lds"):
-            continue
-        if any(w in ABLATE and l.startswith("global_load_lds") and f"%[{op}" in l
-               for w, op in (("copyw", "vw"), ("copyt", "va"), ("copys", "vs]"))):
-            continue
-        if "read" in ABLATE and l.startswith("ds_read_b128") and "%[w" in l:
-            continue
-        if "roll" in ABLATE and l.startswith("ds_read_b128") and "%[a" in l and "offset" in l and int(l.split("offset:")[1]) >= 4096:
-            continue
-        if "scread" in ABLATE and (l.startswith("ds_read_u8") or l.startswith("ds_read_b32")):
-            continue
-        if "barrier" in ABLATE and l == "s_barrier":
-            continue
-        if "vmwait" in ABLATE and l.startswith("s_waitcnt vmcnt"):
-            continue
-        if "relaxw" in ABLATE and l.startswith("s_waitcnt vmcnt("):
-            n = int(l.split("(")[1].split(")")[0])
-            if n > 4:
-                l = l.replace(f"vmcnt({n})", f"vmcnt({n + 4})")
-        out.append(l)
-    return out
-
-
 def emit(name, mtw, fuse):
     p = Plan(mtw, fuse)
-    lines = ablated(with_prio(memory_phase(p), prio("mprio"), "s_waitcnt lgkmcnt(0)")
-                    + with_prio(matrix_phase(p), prio("prio", MATRIX_PRIO), "s_waitcnt vmcnt(4)"))
+    lines = memory_phase(p) + with_prio(matrix_phase(p), MATRIX_PRIO, "s_waitcnt vmcnt(4)")
     print_body(name, lines)
     outs = [f'[c{nt}_{mt}_{i}] "+v"(acc[{nt}][{mt}][{i}])' for mt in range(mtw) for nt in range(NT) for i in range(4)]
     outs += [f'[va{i}] "+v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "+v"(vw[{i}])' for i in range(4)]
@@ -328,7 +279,7 @@ def mx_memory_phase(p):
     for mt in range(p.mtw):
         L.append(f"ds_read_u8 v{p.sfa + mt}, %[sfa{mt}]")
     # the group's own token fragments and token scales (they live in its token slots) may still be out at the barrier
-    L.append("s_waitcnt lgkmcnt(0)" if "latebar" in ABLATE else f"s_waitcnt lgkmcnt({4 + p.mtw})")
+    L.append(f"s_waitcnt lgkmcnt({4 + p.mtw})")
     L.append(f"s_waitcnt vmcnt({p.ntc + 5}) ; explicit")
     L.append("s_barrier")
     L.append("s_waitcnt lgkmcnt(0)")
@@ -369,7 +320,7 @@ def mx_bookkeeping(p):
 
 def mx_matrix_phase(p):
     L = []
-    atoms, late = mx_bookkeeping(p) if "nobook" not in ABLATE else ([], [])
+    atoms, late = mx_bookkeeping(p)
     total = p.mtw * NT
     last_roll = (p.mtw - 3) * NT      # MFMA behind which the last rolling token read issues
     for j in range(total):
@@ -395,8 +346,7 @@ def mx_matrix_phase(p):
 
 def emit_mx(name, mtw, fuse=False):
     p = MxPlan(mtw, fuse)
-    lines = ablated(with_prio(mx_memory_phase(p), prio("mprio"), "s_waitcnt lgkmcnt(0)")
-                    + with_prio(mx_matrix_phase(p), prio("prio", MATRIX_PRIO), "s_waitcnt vmcnt(4)"))
+    lines = mx_memory_phase(p) + with_prio(mx_matrix_phase(p), MATRIX_PRIO, "s_waitcnt vmcnt(4)")
     print_body(name, lines)
     outs = [f'[c{nt}_{mt}] "+v"(acc[{nt}][{mt}])' for mt in range(mtw) for nt in range(NT)]
     outs += [f'[va{i}] "+v"(va[{i}])' for i in range(p.ntc)] + [f'[vw{i}] "+v"(vw[{i}])' for i in range(4)]
@@ -413,8 +363,6 @@ def emit_mx(name, mtw, fuse=False):
 
 
 def main():
-    for a in sys.argv[1:]:
-        ABLATE.add(a)
     print("// Generated by gen_pp_phase.py; do not edit.")
     print("#pragma once")
     for mtw in (4, 6):

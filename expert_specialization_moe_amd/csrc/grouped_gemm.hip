@@ -39,19 +39,9 @@
 
 #include "gemm_args.h"
 #include "mx_scale.h"
-#ifdef ESMOE_PP_HEADER
-#include ESMOE_PP_HEADER
-#else
 #include "pp_phase.h"
-#endif
 #include "schedule.h"
 #include "swiglu.h"
-
-// 1: the hand-scheduled tall tiles copy weight rows that only one tile reads with the non-temporal hint, 0: never
-// (for measurements)
-#ifndef ESMOE_PP_NT
-#define ESMOE_PP_NT 1
-#endif
 
 namespace esmoe {
 
@@ -712,7 +702,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int erow, in
 }
 
 // ---------------------------------------------------------------------------------------------
-// Tall fp8-blockwise tiles (MT = 8 or 12, K a multiple of 512): the K block is one hand-scheduled statement
+// Tall fp8-blockwise tiles (MT = 8 or 12, any K): the K block is one hand-scheduled statement
 // (pp_phase.h, written by gen_pp_phase.py) and the ring is split by operand.
 //
 //   LDS   [0, 96 KB)            weight stages, 3 slots of 256 rows x 128 B, shared by the two groups
@@ -727,8 +717,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, int e, int erow, in
 // slot is refilled with stage kb + 3 from 2kb + 2 on, three or more intervals before 2kb + 6; a group's token stage
 // kb is read in its memory and matrix phase of kb and refilled in its memory phase of kb + 1 with stage kb + 2.
 template <int MT, bool FUSE>
-__device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int erow, int M, int m0, int n0, uint8_t* lds,
-                                             uint32_t* timeline = nullptr) {
+__device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int erow, int M, int m0, int n0, uint8_t* lds) {
   static_assert(MT == 8 || MT == 12, "hand-scheduled K block: 128- and 192-row tiles");
   constexpr int MTW = MT / 2, NTW = 4, BM = MT * 16, GR = MTW * 16;
   constexpr int kTCopies = MTW / 2;                 // token copies per wavefront and K block (8 rows each)
@@ -782,13 +771,8 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int erow,
     const int grow = trow > a_last ? a_last : trow;
     vs[q] = (uint32_t)grow * (uint32_t)KB * 4 + ((lane & 3) < KB ? (lane & 3) : KB - 1) * 4;
   }
-#ifdef ESMOE_EXP_SAMEPANEL   // timing experiment (results wrong): every tall tile of an expert reads the same operand panels
-  const uint8_t* a_ptr = (const uint8_t*)g.a + (row_base + 0) * K - kBias;
-  const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + 0) * K - kBias;
-#else
   const uint8_t* a_ptr = (const uint8_t*)g.a + (row_base + m0) * K - kBias;
   const uint8_t* w_ptr = (const uint8_t*)g.b + ((long)e * N + (FUSE ? 0 : n0)) * K - kBias;
-#endif
   const uint8_t* sa_ptr = (const uint8_t*)(g.sa + (row_base + m0) * KB);
   const uint32_t t_dst = lds0 + kTBase + grp * 2 * kTSlot + wj * kTCopies * 1024;   // + slot * kTSlot
   const uint32_t w_dst = lds0 + wave * 4096;                                        // + slot * kWSlot
@@ -836,13 +820,10 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int erow,
   block_barrier();
   if (grp == 1) block_barrier();
 
-#ifdef ESMOE_TIMELINE
-  const uint64_t tl_r0 = __builtin_amdgcn_s_memrealtime(), tl_c0 = __builtin_amdgcn_s_memtime();
-#endif
   // Weight rows that no other tile reads (the expert is one tile high) are copied with the non-temporal hint, so
   // that their stream leaves L2 to the operands that are shared.  One loop per form: a statement of each kind on
   // alternative paths of one loop would make the compiler shuffle the accumulators between them.
-  const bool w_once = ESMOE_PP_NT && m0 == 0 && M <= BM;
+  const bool w_once = m0 == 0 && M <= BM;
   // The token slot, the weight slot and the copies' source offsets are in/out operands of the statement, which advances
   // them behind its MFMAs (gen_pp_phase.py, bookkeeping); the values below are those of K block 0: token slot 0 is read
   // and slot 1 filled, weight slot 0 is read and slot 2 filled, the copies fetch token stage 1 and weight stage 2.  What
@@ -886,13 +867,6 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int erow,
     }
   };
   if (w_once) k_loop(std::true_type{}); else k_loop(std::false_type{});
-#ifdef ESMOE_TIMELINE
-  if (timeline && tid == 0) {   // debug build: K loop start and end (100 MHz ticks), its length in shader clocks
-    timeline[4] = (uint32_t)tl_r0;
-    timeline[5] = (uint32_t)__builtin_amdgcn_s_memrealtime();
-    timeline[6] = (uint32_t)(__builtin_amdgcn_s_memtime() - tl_c0);
-  }
-#endif
   // the copies past the last K block (they fetched it again) must have landed before anything reuses the ring
   wait_vmcnt<0>();
   if (grp == 0) block_barrier();
@@ -909,8 +883,7 @@ __device__ __forceinline__ void gemm_tile_pp(const GemmArgs& g, int e, int erow,
 // A tile may start in the middle of a 128-row scale tile (full tiles are 192 rows): a lane finds the scale dword of
 // its row from the row's position inside the two tiles that were fetched for its group.
 template <int MT, bool FUSE>
-__device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int erow, int ebso, int M, int m0, int n0, uint8_t* lds,
-                                                uint32_t* timeline = nullptr) {
+__device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int erow, int ebso, int M, int m0, int n0, uint8_t* lds) {
   static_assert(MT == 8 || MT == 12, "hand-scheduled K block: 128- and 192-row tiles");
   constexpr int MTW = MT / 2, NTW = 4, BM = MT * 16, GR = MTW * 16;
   constexpr int kTCopies = MTW / 2;
@@ -1024,10 +997,7 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int er
   block_barrier();
   if (grp == 1) block_barrier();
 
-#ifdef ESMOE_TIMELINE
-  const uint64_t tl_r0 = __builtin_amdgcn_s_memrealtime(), tl_c0 = __builtin_amdgcn_s_memtime();
-#endif
-  const bool w_once = ESMOE_PP_NT && m0 == 0 && M <= BM;   // nobody else reads these weight rows: non-temporal copies (see gemm_tile_pp)
+  const bool w_once = m0 == 0 && M <= BM;   // nobody else reads these weight rows: non-temporal copies (see gemm_tile_pp)
   // Everything that changes from one K block to the next is an in/out operand of the statement, which advances it
   // behind its MFMAs (gen_pp_phase.py, mx_bookkeeping); the values below are those of K block 0: token slot 0 is
   // read and slot 1 filled, weight slot 0 is read and slot 2 filled, the copies fetch token stage 1 and weight stage 2.
@@ -1060,13 +1030,6 @@ __device__ __forceinline__ void gemm_tile_pp_mx(const GemmArgs& g, int e, int er
     }
   };
   if (w_once) k_loop(std::true_type{}); else k_loop(std::false_type{});
-#ifdef ESMOE_TIMELINE
-  if (timeline && tid == 0) {
-    timeline[4] = (uint32_t)tl_r0;
-    timeline[5] = (uint32_t)__builtin_amdgcn_s_memrealtime();
-    timeline[6] = (uint32_t)(__builtin_amdgcn_s_memtime() - tl_c0);
-  }
-#endif
   wait_vmcnt<0>();
   if (grp == 0) block_barrier();
   block_barrier();
@@ -1241,19 +1204,6 @@ __device__ __forceinline__ void self_schedule(const GemmArgs& g, uint8_t* lds, i
   __syncthreads();
 }
 
-// Heights whose fp8-blockwise tiles run the hand-scheduled K block of gemm_tile_pp (bit 0: 128 rows, bit 1: 192 rows).
-#ifndef ESMOE_PP_HEIGHTS
-#define ESMOE_PP_HEIGHTS 3
-#endif
-// The same for mxfp8 tiles (gemm_tile_pp_mx).
-#ifndef ESMOE_PPX_HEIGHTS
-#define ESMOE_PPX_HEIGHTS 3
-#endif
-// Tile heights (MT * 16 rows) compiled into the persistent kernel.
-#ifndef ESMOE_VARIANTS
-#define ESMOE_VARIANTS ESMOE_CASE(1) ESMOE_CASE(2) ESMOE_CASE(4)
-#endif
-
 template <bool MX, bool FUSE>
 __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kLdsBytes];
@@ -1269,9 +1219,6 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     lsplit = ws[kWsLightSplit];
     lshare = ws[kWsLightShare];
   }
-#define ESMOE_CASE(MT_) \
-  case (MT_): gemm_tile<MT_, MX, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
-
   // Workgroup i runs on XCD i % 8 (HW_REG_XCC_ID = 20, bits [3:0], says so directly).  Of every 32 workgroups
   // of an XCD the last `light_share` start on the light items, the others on the heavy tickets; either kind
   // moves on to the other when its own is exhausted.
@@ -1287,10 +1234,6 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
 #pragma unroll
   for (int x = 0; x < kXcds; x++)
     if (x >= hblocks) dead |= 1 << x;
-#ifdef ESMOE_TIMELINE
-  int tl_n = 0;
-  if (threadIdx.x == 0) ((uint32_t*)ws)[4096 + blockIdx.x * 256] = 0;
-#endif
   for (;;) {
     const bool light = (phase == 0) == light_first;
     const int xq = (xcd + q) & (kXcds - 1);
@@ -1305,13 +1248,7 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
     __syncthreads();
     const int ticket = __builtin_amdgcn_readfirstlane(s_item);
     const int kind = light ? kRecItem : kRecBlock;
-#ifdef ESMOE_TIMELINE
-    // (the debug build's extra code keeps the compiler from seeing that this is wave-uniform, and the copies need
-    // their base pointers in scalar registers)
-    const int v = __builtin_amdgcn_readfirstlane(light ? ticket : sched_ticket_block(xq, ticket));
-#else
     const int v = light ? ticket : sched_ticket_block(xq, ticket);
-#endif
     if (v >= (light ? ltotal : hblocks)) {   // this queue is exhausted: see which others are
       dead |= 1 << (light ? 8 : xq);
       __syncthreads();                        // s_item and s_counters are rewritten next
@@ -1364,63 +1301,27 @@ __global__ void __launch_bounds__(kThreads) grouped_gemm_kernel(GemmArgs g) {
       __syncthreads();
       continue;
     }
-#ifdef ESMOE_TIMELINE
-    const uint64_t tl_t0 = __builtin_amdgcn_s_memrealtime();
-#define ESMOE_TL_PTR (tl_n < 31 ? (uint32_t*)ws + 4096 + blockIdx.x * 256 + 8 + tl_n * 8 : nullptr)
-#else
-#define ESMOE_TL_PTR nullptr
-#endif
-    // tall fp8-blockwise tiles take the hand-scheduled K block when the scale chunks fit K (a multiple of 512)
-    bool hand_scheduled = false;
-    if constexpr (MX) {
-      if ((ESMOE_PPX_HEIGHTS & 2) && t.mt == 12) {
-        gemm_tile_pp_mx<12, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
-        hand_scheduled = true;
-      } else if ((ESMOE_PPX_HEIGHTS & 1) && t.mt == 8) {
-        gemm_tile_pp_mx<8, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
-        hand_scheduled = true;
+    // Tile heights (MT * 16 rows): 8 and 12 are the tall tiles with the hand-scheduled K block, 1, 2 and 4 the short
+    // ones, also as 128-column halves.  The host refuses a policy that asks for any other height (launch_gemm), so
+    // every ticket finds its tile function here.
+    if (t.mt == 12) {
+      if constexpr (MX) gemm_tile_pp_mx<12, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds);
+      else gemm_tile_pp<12, FUSE>(g, e, erow, M, t.m0, t.n0, lds);
+    } else if (t.mt == 8) {
+      if constexpr (MX) gemm_tile_pp_mx<8, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds);
+      else gemm_tile_pp<8, FUSE>(g, e, erow, M, t.m0, t.n0, lds);
+    } else if (!FUSE && t.nt == 2) {
+      if constexpr (!FUSE) {
+        if (t.mt == 1) gemm_tile<1, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds);
+        else if (t.mt == 2) gemm_tile<2, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds);
+        else gemm_tile<4, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds);
       }
+    } else {
+      if (t.mt == 1) gemm_tile<1, MX, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds);
+      else if (t.mt == 2) gemm_tile<2, MX, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds);
+      else gemm_tile<4, MX, FUSE>(g, e, erow, ebso, M, t.m0, t.n0, lds);
     }
-    if constexpr (!MX) {
-      if ((ESMOE_PP_HEIGHTS & 2) && t.mt == 12) {
-        gemm_tile_pp<12, FUSE>(g, e, erow, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
-        hand_scheduled = true;
-      } else if ((ESMOE_PP_HEIGHTS & 1) && t.mt == 8) {
-        gemm_tile_pp<8, FUSE>(g, e, erow, M, t.m0, t.n0, lds, ESMOE_TL_PTR);
-        hand_scheduled = true;
-      }
-    }
-    if (!hand_scheduled) {
-      if (!FUSE && t.nt == 2) {
-        if constexpr (!FUSE) {
-          switch (t.mt) {
-            case 1: gemm_tile<1, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
-            case 2: gemm_tile<2, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
-            case 4: gemm_tile<4, MX, false, 128>(g, e, erow, ebso, M, t.m0, t.n0, lds); break;
-            default: break;
-          }
-        }
-      } else {
-        switch (t.mt) {
-          ESMOE_VARIANTS
-          default: break;
-        }
-      }
-    }
-#ifdef ESMOE_TIMELINE
-    // debug build only: (start, end, kind, position) of this workgroup's first 31 tiles, in 100 MHz ticks, 8 words
-    // per tile, into a caller-provided oversize workspace from word 4096 on
-    if (threadIdx.x == 0 && tl_n < 31) {
-      uint32_t* tl = (uint32_t*)ws + 4096 + blockIdx.x * 256;
-      tl[8 + tl_n * 8 + 0] = (uint32_t)tl_t0;
-      tl[8 + tl_n * 8 + 1] = (uint32_t)__builtin_amdgcn_s_memrealtime();
-      tl[8 + tl_n * 8 + 2] = (uint32_t)(t.mt | (light ? 256 : 0) | (xcd << 12) | (e << 16));
-      tl[8 + tl_n * 8 + 3] = (uint32_t)(t.m0 / 16) | ((uint32_t)(t.n0 / 256) << 16);
-      tl[0] = ++tl_n;
-    }
-#endif
   }
-#undef ESMOE_CASE
   // The last workgroup to leave zeroes the hand-out counters (nobody draws any more: every workgroup counts itself
   // out after its last draw), so a workspace that held zero counters before the launch holds them again after it.
   if (threadIdx.x == 0) {

@@ -21,11 +21,11 @@
 
 namespace esmoe {
 
-// Row-tile heights are MT * 16 rows with MT in {1, 2, 4, 8, 12, 16}; a workgroup tile
+// Row-tile heights are MT * 16 rows with MT in {1, 2, 4, 8, 12} (sched_valid_mt); a workgroup tile
 // is (MT * 16) rows by 256 columns.
 struct SchedPolicy {
   int force_mt;   // 0 = choose per expert; else every tile uses this MT
-  int big_mt;     // MT of the full tiles of a many-row expert (8, 12 or 16)
+  int big_mt;     // MT of the full tiles of a many-row expert (8 or 12)
   int order;      // 0: heavy experts by rows ascending, light ones descending (sched_order_key); 1: expert index order;
                   // 2: most rows first for both kinds
   int light_share;  // workgroups (of every 32) that start on the light items; -1 = from the cost estimate
@@ -39,7 +39,10 @@ struct TileCoord {
   int n0;  // first column
 };
 
-// Smallest tile height of the menu {1, 2, 4, 8, 12, 16} (x16 rows) that covers `rows`, at most max_mt.
+// The tile heights the kernels are compiled for.
+ESMOE_HD bool sched_valid_mt(int mt) { return mt == 1 || mt == 2 || mt == 4 || mt == 8 || mt == 12; }
+
+// Smallest tile height of the menu {1, 2, 4, 8, 12} (x16 rows) that covers `rows`, at most max_mt.
 ESMOE_HD int sched_cover_mt(int rows, int max_mt) {
   const int need = (rows + 15) / 16;
   int mt = 1;
@@ -47,7 +50,6 @@ ESMOE_HD int sched_cover_mt(int rows, int max_mt) {
   if (need > 2) mt = 4;
   if (need > 4) mt = 8;
   if (need > 8) mt = 12;
-  if (need > 12) mt = 16;
   return mt < max_mt ? mt : max_mt;
 }
 
