@@ -20,10 +20,10 @@ import torch
 # this script (summaries under profiles/), each scaled by the same counter's reading for a 1 GiB copy kernel.
 # Keyed by (config, op); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    ("c1", "gemm"): 1.546e9,     # FETCH 728,712.7 x 2.000 KiB + WRITE 52,745.4 x 1.000 KiB
-    ("c2", "gemm"): 4.486e8,     # FETCH 217,244.4 x 2.000 KiB + WRITE 3,630.7 x 1.000 KiB
-    ("c4", "gemm"): 1.455e9,     # FETCH 677,660.2 x 2.000 KiB + WRITE 65,715.8 x 1.000 KiB
-    ("c4", "quant"): 1.786e8,    # FETCH 57,399.0 x 2.000 KiB + WRITE 59,584.0 x 1.000 KiB
+    ("c1", "gemm"): 1.546e9,     # FETCH 728,218.9 x 2.000 KiB + WRITE 52,804.0 x 1.000 KiB
+    ("c2", "gemm"): 4.485e8,     # FETCH 217,195.5 x 2.000 KiB + WRITE 3,643.1 x 1.000 KiB
+    ("c4", "gemm"): 1.452e9,     # FETCH 676,216.6 x 2.000 KiB + WRITE 65,709.2 x 1.000 KiB
+    ("c4", "quant"): 1.785e8,    # FETCH 57,378.0 x 2.000 KiB + WRITE 59,584.5 x 1.000 KiB
 }
 
 
