@@ -165,6 +165,9 @@ __global__ void __launch_bounds__(quant_threads<SWIGLU>()) __attribute__((amdgpu
     int codes = live ? code : 0;
     codes |= dpp_i32<0x104>(codes) << 8;     // from lane + 4 of the 16-lane row
     codes |= dpp_i32<0x108>(codes) << 16;    // from lane + 8
+    // (the exchanges have to run with every lane active: the empty statement keeps the compiler from moving them into
+    // the store's branch below, where their source lanes would be switched off and read as 0)
+    asm volatile("" : "+v"(codes));
     unit[j] = codes;
   }
   if ((sub & 15) == 0 && col_ok)
